@@ -53,15 +53,18 @@ class Model(Part):
             self.blocks.append(self.attach(f"layers.{i}", block))
         self.attach("norm", build.make(spec.norm, dim=spec.hidden))
         self.attach("lm_head", build.make(spec.head, vocab=spec.vocab, hidden=spec.hidden, embed=self.embed))
+        self._keeps_origin = any(b.reads_origin for b in self.blocks)
         self.sites = [Site(run=at, layer=r.layer, writes=r.reads is None, owner=r.reads)
                       for at, r in enumerate(spec.order)]
 
     def state_decls(self) -> list[list[PagedState | SlotState]]:
-        """Per run, what its mixer keeps between steps (empty for a run that reads another's cache)."""
+        """Per run, what its layer keeps between steps (empty for a run that reads another's cache): what the block
+        declares itself (a block with state beside its mixer's), else what its mixer declares."""
         out = []
         for site in self.sites:
-            mixer = getattr(self.blocks[site.layer], "mixer", None)
-            out.append(list(mixer.state()) if mixer is not None and site.writes else [])
+            block = self.blocks[site.layer]
+            keeper = block if block.state() else getattr(block, "mixer", None)
+            out.append(list(keeper.state()) if keeper is not None and site.writes else [])
         return out
 
     def cut(self, start: int, count: int) -> int:
@@ -74,7 +77,7 @@ class Model(Part):
     def trunk(self, step) -> tuple[torch.Tensor, torch.Tensor | None]:
         """The residual stream after every run, as (h, delta) with h + delta the stream [T, hidden]."""
         h, stats = self.embed(step.token_ids, step.token_take, want_stats=True)
-        stream = Stream(h, stats=stats)
+        stream = Stream(h, stats=stats, origin=h if self._keeps_origin else None)
         for site in self.sites:
             stream = self.blocks[site.layer](stream, step, site)
         return stream.h, stream.delta

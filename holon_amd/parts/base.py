@@ -24,9 +24,9 @@ class ParamDecl:
     """A tensor a part owns. `kind`: "model" is kept in the engine's dtype; "float32" is kept in 32-bit whatever the
     engine's dtype; "int32" is an integer table."""
 
-    shape: tuple[int, ...]
+    shape: tuple[int, ...]                        # a size of -1 is whatever the checkpoint's tensor has there
     kind: str = MODEL
-    init: str = "linear"                          # how random weights draw it: linear | norm
+    init: str = "linear"                          # how random weights draw it: linear | norm | unit | tap | zero
 
 
 @dataclasses.dataclass(frozen=True)
@@ -82,6 +82,8 @@ class Stream:
     h: torch.Tensor
     delta: "torch.Tensor | PartialSums | None" = None
     stats: torch.Tensor | None = None
+    origin: torch.Tensor | None = None            # the embedding's rows, for a model with a block that reads them
+                                                  # again (`Part.reads_origin`); nobody writes into this tensor
 
 
 @dataclasses.dataclass
@@ -104,6 +106,7 @@ class Build:
 class Part:
     """Base of all parts. Subclasses call `declare` for tensors and `attach` for sub-parts in `__init__`."""
 
+    reads_origin = False      # a block that needs the embedding's rows beside the stream (`Stream.origin`)
     adds_residual = False     # its forward accepts `residual=h`: it may add its result into h and return None
     graph_safe = False        # True: a captured step may be replayed over it. Its forward then reads nothing on the
                               # host that changes from step to step (no `step.h_*`, no `.item()`, no shapes that depend

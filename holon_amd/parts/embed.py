@@ -29,13 +29,16 @@ class Embedding(EmbedPart):
 
 @register_part("head", "linear")
 class LMHead(Part):
-    """Logits in float32. A tied head owns no tensor: it reads the embedding's."""
+    """Logits in float32, optionally squashed into (-softcap, softcap). A tied head owns no tensor: it reads the
+    embedding's."""
 
     graph_safe = True
 
-    def __init__(self, build: Build, *, vocab: int, hidden: int, tied: bool, embed: Embedding) -> None:
+    def __init__(self, build: Build, *, vocab: int, hidden: int, tied: bool, embed: Embedding,
+                 softcap: float | None = None) -> None:
         super().__init__(build)
         self.tied = tied
+        self.softcap = float(softcap) if softcap else None      # logits <- cap * tanh(logits / cap)
         self._embed = [embed]                     # in a list: the embedding part keeps the one owner of the tensor
         self.tiled: torch.Tensor | None = None
         if not tied:
@@ -52,6 +55,7 @@ class LMHead(Part):
         return [self.tiled] if self.tiled is not None else []
 
     def forward(self, h: torch.Tensor) -> torch.Tensor:
-        return self.kernels.linear(h, self._weight(), torch.float32, self.tiled)
+        logits = self.kernels.linear(h, self._weight(), torch.float32, self.tiled)
+        return logits if self.softcap is None else self.kernels.softcap(logits, self.softcap)
 
     __call__ = forward

@@ -95,3 +95,28 @@ class GQA(Part):
         return self.o_proj(out.view(t, hq * d), residual=residual)
 
     __call__ = forward
+
+
+@register_part("mixer", "parallel")
+class ParallelMixers(Part):
+    """Two mixers side by side that read the same input; the result is left_scale * left + right_scale * right. The
+    two results are handed on as terms with their scales (`Pending`) to a block whose residual add takes them in one
+    kernel; `left` and `right` are any registered mixers, each keeping its state under its own name."""
+
+    graph_safe = True
+
+    def __init__(self, build: Build, *, left: PartRef, right: PartRef, left_scale: float, right_scale: float,
+                 hidden: int, layer: int) -> None:
+        super().__init__(build)
+        self.left_scale, self.right_scale = float(left_scale), float(right_scale)
+        self.attach("left", build.make(left, hidden=hidden, layer=layer, name="left"))
+        self.attach("right", build.make(right, hidden=hidden, layer=layer, name="right"))
+
+    def state(self):
+        return list(self.left.state()) + list(self.right.state())
+
+    def forward(self, x, step, site):
+        from .stream32 import Pending
+        return Pending([(self.left(x, step, site), self.left_scale), (self.right(x, step, site), self.right_scale)])
+
+    __call__ = forward

@@ -3,6 +3,8 @@ std/holon_std/ops/units.py:38-63 (`Rope`), formula std/holon_std/ops/reference.p
 std/holon_std/ops/kernels.py:7-12."""
 from __future__ import annotations
 
+import math
+
 import torch
 
 from ..registry import register_part
@@ -40,6 +42,43 @@ class Rope(Part):
 
     def fusion(self) -> dict | None:
         return {"position": "rope", "table": self.table}
+
+
+def banded_frequencies(rotary_dim: int, base: float, scaling: dict | None) -> torch.Tensor:
+    """f_i = base^(-2i/rotary_dim) for the rotary_dim/2 pairs, float32 (computed in float64, rounded once). With
+    `scaling` = {factor, low, high, original}, by wavelength l = 2 pi / f: waves shorter than original/high keep f,
+    waves longer than original/low turn `factor` times slower, and between the two the slow and the plain frequency
+    are blended linearly in original/l (the long-context rescaling of Llama 3.1)."""
+    i = torch.arange(rotary_dim // 2, dtype=torch.float64)
+    f = torch.as_tensor(float(base), dtype=torch.float64) ** (-2.0 * i / rotary_dim)
+    if scaling:
+        factor, low, high, original = (float(scaling[k]) for k in ("factor", "low", "high", "original"))
+        wave = 2 * math.pi / f
+        blend = ((original / wave - low) / (high - low)) if high != low else torch.ones_like(f)
+        mid = (1 - blend) * f / factor + blend * f
+        f = torch.where(wave < original / high, f, torch.where(wave > original / low, f / factor, mid))
+    return f.to(torch.float32)
+
+
+@register_part("position", "rope_banded")
+class BandedRope(Rope):
+    """Rotary embedding on the first `rotary_dim` dimensions of a head, half-split pairing, with frequencies that may
+    be rescaled in bands of wavelength (`scaling`, given as a dict or as its sorted items). Angles are the float32
+    product of position and frequency."""
+
+    graph_safe = True
+
+    def __init__(self, build: Build, *, theta: float, head_dim: int, rotary_dim: int | None = None,
+                 scaling=None) -> None:
+        Part.__init__(self, build)
+        self.theta, self.head_dim = float(theta), head_dim
+        self.rotary_dim = head_dim if rotary_dim is None else int(rotary_dim)
+        if self.rotary_dim % 2 or not 0 < self.rotary_dim <= head_dim:
+            raise ValueError(f"rotary_dim {self.rotary_dim} must be even and within head_dim {head_dim}")
+        self.scaling = dict(scaling) if scaling else None
+        freqs = banded_frequencies(self.rotary_dim, self.theta, self.scaling)
+        angles = torch.arange(build.max_model_len, dtype=torch.float32)[:, None] * freqs[None, :]
+        self.table = torch.cat((angles.cos(), angles.sin()), dim=-1).contiguous().to(build.device)
 
 
 @register_part("position", "none")

@@ -51,11 +51,11 @@ def architectures() -> list[str]:
 
 
 def resolve(config_json: Mapping[str, Any], generation: Mapping[str, Any] | None = None) -> tuple[Any, ModelSpec]:
-    """config.json to (typed configuration, model spec), by `architectures[0]`
+    """config.json to (typed configuration, model spec), by `architectures[0]` (or the one name in `architecture`)
     (core/holon/core/assembly.py:28-31)."""
-    names = config_json.get("architectures")
+    names = config_json.get("architectures") or ([config_json["architecture"]] if config_json.get("architecture") else None)
     if not names:
-        raise RegistryError("config.json has no `architectures`")
+        raise RegistryError("config.json has no `architectures` (nor `architecture`)")
     arch = architecture(names[0])
     cfg = arch.config.from_dict(config_json, generation)
     return cfg, arch.recipe(cfg)

@@ -42,7 +42,7 @@ class LayerSpec:
 
     block: PartRef
     mixer: PartRef
-    ffn: PartRef
+    ffn: PartRef | None                          # None: the layer has no feed-forward (for blocks that allow it)
     norm: PartRef
 
 
@@ -108,7 +108,8 @@ class ModelSpec:
     def identity(self) -> str:
         """A hash of everything that decides the computation (core/holon/api/terms.py:98-100)."""
         doc = {"hidden": self.hidden, "vocab": self.vocab,
-               "layers": [[getattr(l, f).canonical() for f in ("block", "mixer", "ffn", "norm")] for l in self.layers],
+               "layers": [[getattr(l, f).canonical() if getattr(l, f) is not None else None
+                           for f in ("block", "mixer", "ffn", "norm")] for l in self.layers],
                "order": [[r.layer, r.reads] for r in self.order],
                "embed": self.embed.canonical(), "norm": self.norm.canonical(), "head": self.head.canonical()}
         return hashlib.sha256(json.dumps(doc, sort_keys=True).encode()).hexdigest()[:16]

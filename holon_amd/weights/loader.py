@@ -123,8 +123,8 @@ def load_weights(model: Part, spec: ModelSpec, folder: str | pathlib.Path, devic
                     other.append(f"tensors {where[found][1]} and {name} both fill {path}")
                     continue
                 got = tuple(f.get_slice(name).get_shape())
-                if got != want:
-                    wrong.append((name, got, want))
+                if len(got) != len(want) or any(w not in (-1, g) for g, w in zip(got, want)):
+                    wrong.append((name, got, want))               # (a declared size of -1 takes the tensor's)
                 where[found] = (file, name)
     stacked = {path for path, index in where if index is not None}
     for path, (_, _, decl) in params.items():

@@ -1,7 +1,9 @@
 """Random weights from a configuration and a seed: written as a model folder, or put straight into a built model.
 
 Each tensor is drawn from its own generator, seeded by (seed, checkpoint tensor name), so the values do not depend on
-the order of creation. Projections and the embedding are N(0, 0.02); norm weights are 1 + N(0, 0.1). Values are
+the order of creation. Projections and the embedding are N(0, 0.02); norm weights are 1 + N(0, 0.1); a parameter may
+ask for another law (`ParamDecl.init`): `unit` is uniform in [0, 1), `tap` N(0, 0.3) (a short filter's taps), `zero`
+N(0, 0.5) (offsets around zero that feed an exponential or a sigmoid). Values are
 rounded to bfloat16 before they are stored, so the 32-bit and the bfloat16 model of one folder hold the same numbers.
 """
 from __future__ import annotations
@@ -19,7 +21,7 @@ from ..parts.base import INT32, Build, ParamDecl
 from ..registry import resolve
 from .loader import checkpoint_names, finalize, param_dtype
 
-LINEAR_STD, NORM_STD = 0.02, 0.1
+LINEAR_STD, NORM_STD, TAP_STD, ZERO_STD = 0.02, 0.1, 0.3, 0.5
 
 
 def tensor_seed(seed: int, name: str) -> int:
@@ -30,9 +32,16 @@ def random_tensor(name: str, decl: ParamDecl, seed: int, device: torch.device | 
     """float32 values (bfloat16-representable) of tensor `name`."""
     if decl.kind == INT32:
         raise NotImplementedError(f"{name}: no rule to draw an integer table")
+    if any(s < 0 for s in decl.shape):
+        raise ValueError(f"{name}: shape {decl.shape} has a size that only a checkpoint gives; name it in the "
+                         "configuration to draw random weights")
     g = torch.Generator(device=device).manual_seed(tensor_seed(seed, name))
-    x = torch.randn(decl.shape, generator=g, device=device, dtype=torch.float32)
-    x = 1 + NORM_STD * x if decl.init == "norm" else LINEAR_STD * x
+    if decl.init == "unit":
+        x = torch.rand(decl.shape, generator=g, device=device, dtype=torch.float32)
+    else:
+        x = torch.randn(decl.shape, generator=g, device=device, dtype=torch.float32)
+        x = 1 + NORM_STD * x if decl.init == "norm" else \
+            {"linear": LINEAR_STD, "tap": TAP_STD, "zero": ZERO_STD}[decl.init] * x
     return x.bfloat16().float()
 
 
