@@ -167,6 +167,62 @@ int holon_scatter_rows(int32_t* dst, const int32_t* idx, const int32_t* src, int
 int holon_logprobs(const float* logits, const int32_t* tokens, int rows, int vocab, int k, float* token_lp,
                    int32_t* top_ids, float* top_lp, void* stream);
 
+// -- a float32 residual stream (stream32.hip) ---------------------------------------------------------------------------
+// y[i] = x[i] as float32 (x float32 or bfloat16): a new copy.
+int holon_widen_rows(const void* x, float* y, int64_t n, int dtype, void* stream);
+// x32 [rows, dim] += s1 d1 + s2 d2 in place (d1, d2 nullable, each float32 or bfloat16 by dt1, dt2); then, with
+// weight and y (both or neither): y = (x - mean) / sqrt(var + eps) * weight, weight and y of dtype dt_out.
+int holon_stream_norm(float* x32, const void* d1, float s1, int dt1, const void* d2, float s2, int dt2,
+                      const void* weight, void* y, int64_t rows, int dim, float eps, int dt_out, void* stream);
+// y [rows, w1 + w2] = [x32 | origin] in dt_out.
+int holon_pair_rows(const float* x32, const void* origin, void* y, int64_t rows, int w1, int w2, int dt_origin,
+                    int dt_out, void* stream);
+// logits <- cap * tanh(logits / cap) in place.
+int holon_softcap(float* logits, int64_t n, float cap, void* stream);
+
+// -- recurrent mixers (recurrent.hip); rows are ranges query_start[b] .. query_start[b + 1] of the flat tokens ----------
+// y_t[c] = act(sum_j w[c, j] x_(t - taps + 1 + j)[c] (+ x_t[c])); state [state_slots, taps - 1, channels] holds each
+// request's last inputs (ignored by a row that starts at 0) and takes the row's last ones afterwards.
+int holon_causal_conv(const void* x, const void* w, void* state, void* y, const int32_t* slots, const int32_t* starts,
+                      const int32_t* query_start, const int32_t* token_row, int tokens, int rows, int channels, int taps,
+                      int state_slots, int add_input, int act, int dtype, void* stream);
+// From filtered q, k, v [T, 2 G D + H V] and the projections ab [T, 2 H]: unit q (times D^-0.5) and k [T, G, D],
+// beta = sigmoid(b), g = exp(-exp(a_log) softplus(a + dt_bias)) [T, H]; all outputs float32.
+int holon_delta_prepare(const void* qkv, const void* ab, const float* a_log, const float* dt_bias, float* qn, float* kn,
+                        float* beta, float* g, int tokens, int heads, int kv_heads, int dim, int vdim, int dtype,
+                        void* stream);
+// The gated delta rule over each row's tokens; v = qkv[t, v_offset + h V + j]; state [state_slots, H, D, V] float32.
+int holon_delta_scan(const float* qn, const float* kn, const void* qkv, int qkv_stride, int v_offset, const float* beta,
+                     const float* g, float* state, float* out, const int32_t* slots, const int32_t* starts,
+                     const int32_t* query_start, int rows, int heads, int kv_heads, int dim, int vdim, int state_slots,
+                     int dtype, void* stream);
+// The decayed key-value memory over each row's tokens; r, k, v [T, H D]; w [T, H D] float32; u [H, D];
+// state [state_slots, H, D, D] float32.
+int holon_memory_scan(const void* r, const void* k, const void* v, const float* w, const float* u, float* state,
+                      float* out, const int32_t* slots, const int32_t* starts, const int32_t* query_start, int rows,
+                      int heads, int dim, int state_slots, int dtype, void* stream);
+// y [T, H V] = o / sqrt(mean_V(o^2) + eps) * weight * silu(gate); weight [V], or [H V] with per_head.
+int holon_gated_out(const float* o, const void* gate, const void* weight, void* y, int tokens, int heads, int vdim,
+                    int per_head, float eps, int dtype, void* stream);
+// y [mixes, T, W] = x + (x' - x) mu_s, x' the row of the token before (state [state_slots, W] for a row's first
+// token, zeros for a row that starts at 0); the state then takes each row's last x.
+int holon_shift_mix(const void* x, const void* mu, void* state, void* y, const int32_t* slots, const int32_t* starts,
+                    const int32_t* query_start, const int32_t* token_row, int tokens, int rows, int width, int mixes,
+                    int state_slots, int dtype, void* stream);
+// y [T, C] = exp(-exp(tanh(a [T, R]) w2 [C, R]^T + w0 [C])), float32.
+int holon_decay_lora(const float* a, const void* w2, const float* w0, float* y, int tokens, int channels, int rank,
+                     int dtype, void* stream);
+
+// -- windowed sigmoid attention (sigmoid_attention.hip); a page is keys [Hkv, P, D] then values [Hkv, P, V] ---------------
+int holon_head_prepare(const void* qkv, void* q_out, int tokens, int heads, int kv_heads, int dim, int vdim,
+                       const void* q_weight, const void* k_weight, float eps, const float* table, int rot, int table_rows,
+                       const int32_t* positions, void* pages, const int32_t* write_page, const int32_t* write_off,
+                       int page_size, int num_pages, int dtype, void* stream);
+int holon_sigmoid_attention(const void* q, void* out, const void* pages, const int32_t* table, int table_stride,
+                            const int32_t* slots, const int32_t* token_row, const int32_t* positions, int tokens,
+                            int heads, int kv_heads, int dim, int vdim, int page_size, int num_pages, const float* bias,
+                            float scale, int window, const void* gate, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,397 @@
+// Recurrent mixers: a short causal filter with carried inputs, the gated delta rule, a decayed key-value memory with
+// token shift, and the small float32 steps around them. A step's rows are ranges of its flat tokens
+// (query_start[b] .. query_start[b + 1]), each continuing the state in its request's slot; a row that starts at
+// position 0 starts from zeros whatever the slot holds.
+//
+// The two scans keep, per (row, head), one thread per value column j of the head's matrix S [D, V]: the columns never
+// meet, so a thread carries its D values in registers through the row's tokens; a block is one wave of 64 columns,
+// which shares each token's key and query through LDS. The key size is padded to the next instantiated one with zeros (a zero key writes nothing).
+// Every sum runs over the key index in ascending order.
+#include "common.h"
+#include "holon_hip.h"
+
+namespace {
+
+template <typename T>
+__global__ void causal_conv_kernel(const T* __restrict__ x, const T* __restrict__ w, const T* __restrict__ state,
+                                   T* __restrict__ y, const int32_t* __restrict__ slots,
+                                   const int32_t* __restrict__ starts, const int32_t* __restrict__ query_start,
+                                   const int32_t* __restrict__ token_row, int channels, int taps, int add_input,
+                                   int act) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  const int t = blockIdx.y;
+  if (c >= channels) return;
+  const int b = token_row[t];
+  const int q0 = query_start[b];
+  const int i = t - q0;
+  const bool carried = starts[b] > 0;
+  const T* held = state + (int64_t)slots[b] * (taps - 1) * channels;
+  float acc = 0.f;
+  for (int j = 0; j < taps; ++j) {
+    const int l = i - (taps - 1) + j;
+    float v = 0.f;
+    if (l >= 0) v = Elem<T>::load(x[(int64_t)(q0 + l) * channels + c]);
+    else if (carried) v = Elem<T>::load(held[(int64_t)(taps - 1 + l) * channels + c]);
+    acc += Elem<T>::load(w[(int64_t)c * taps + j]) * v;
+  }
+  if (add_input) acc += Elem<T>::load(x[(int64_t)t * channels + c]);
+  if (act) acc = silu<T>(acc);
+  y[(int64_t)t * channels + c] = Elem<T>::store(acc);
+}
+
+// After the filter has read the old inputs: the slot takes the row's last taps - 1 inputs, oldest first. A thread
+// moves its channel's entries in ascending order and reads only entries at or behind the one it writes.
+template <typename T>
+__global__ void causal_conv_keep_kernel(const T* __restrict__ x, T* __restrict__ state, const int32_t* __restrict__ slots,
+                                        const int32_t* __restrict__ starts, const int32_t* __restrict__ query_start,
+                                        int channels, int taps) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  const int b = blockIdx.y;
+  if (c >= channels) return;
+  const int q0 = query_start[b], n = query_start[b + 1] - q0;
+  const bool carried = starts[b] > 0;
+  T* held = state + (int64_t)slots[b] * (taps - 1) * channels;
+  for (int i = 0; i < taps - 1; ++i) {
+    const int l = n - (taps - 1) + i;
+    T v = Elem<T>::store(0.f);
+    if (l >= 0) v = x[(int64_t)(q0 + l) * channels + c];
+    else if (carried) v = held[(int64_t)(i + n) * channels + c];
+    held[(int64_t)i * channels + c] = v;
+  }
+}
+
+__device__ __forceinline__ float softplus_f(float z) { return z > 20.f ? z : log1pf(expf(z)); }
+
+// One block a token. Waves take the 2 G heads of q and k in turn: unit vectors (q also times D^-0.5); then the step
+// sizes and decays of the H heads.
+template <typename T>
+__global__ void __launch_bounds__(256) delta_prepare_kernel(const T* __restrict__ qkv, const T* __restrict__ ab,
+                                                            const float* __restrict__ a_log,
+                                                            const float* __restrict__ dt_bias, float* __restrict__ qn,
+                                                            float* __restrict__ kn, float* __restrict__ beta,
+                                                            float* __restrict__ g, int heads, int kv_heads, int dim,
+                                                            int vdim) {
+  const int t = blockIdx.x;
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  const int width = 2 * kv_heads * dim + heads * vdim;
+  const T* row = qkv + (int64_t)t * width;
+  for (int idx = wave; idx < 2 * kv_heads; idx += 4) {
+    const bool is_q = idx < kv_heads;
+    const int h = is_q ? idx : idx - kv_heads;
+    const T* src = row + (int64_t)idx * dim;
+    float ss = 0.f;
+    for (int d = lane; d < dim; d += WAVE) {
+      const float v = Elem<T>::load(src[d]);
+      ss += v * v;
+    }
+    ss = wave_sum(ss);
+    const float r = (1.0f / sqrtf(ss + 1e-6f)) * (is_q ? 1.0f / sqrtf((float)dim) : 1.0f);
+    float* dst = (is_q ? qn : kn) + ((int64_t)t * kv_heads + h) * dim;
+    for (int d = lane; d < dim; d += WAVE) dst[d] = Elem<T>::load(src[d]) * r;
+  }
+  for (int h = threadIdx.x; h < heads; h += 256) {
+    const float a = Elem<T>::load(ab[(int64_t)t * 2 * heads + h]);
+    const float b = Elem<T>::load(ab[(int64_t)t * 2 * heads + heads + h]);
+    beta[(int64_t)t * heads + h] = 1.0f / (1.0f + expf(-b));
+    g[(int64_t)t * heads + h] = expf(-expf(a_log[h]) * softplus_f(a + dt_bias[h]));
+  }
+}
+
+// Per (row, head): S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q. Thread j owns column j of S.
+template <int KD, typename T>
+__global__ void __launch_bounds__(WAVE) delta_scan_kernel(const float* __restrict__ qn, const float* __restrict__ kn, const T* __restrict__ qkv,
+                                  int qkv_stride, int v_offset, const float* __restrict__ beta,
+                                  const float* __restrict__ g, float* __restrict__ state, float* __restrict__ out,
+                                  const int32_t* __restrict__ slots, const int32_t* __restrict__ starts,
+                                  const int32_t* __restrict__ query_start, int heads, int kv_heads, int dim, int vdim) {
+  __shared__ float ks[KD], qs[KD];
+  const int b = blockIdx.x, h = blockIdx.y, j = blockIdx.z * WAVE + threadIdx.x;
+  const int hk = h / (heads / kv_heads);
+  const bool active = j < vdim;
+  const int lo = query_start[b], hi = query_start[b + 1];
+  float* held = state + ((int64_t)slots[b] * heads + h) * dim * vdim;
+  const bool carried = starts[b] > 0;
+  float S[KD];
+#pragma unroll
+  for (int i = 0; i < KD; ++i) S[i] = (carried && active && i < dim) ? held[(int64_t)i * vdim + j] : 0.f;
+  for (int t = lo; t < hi; ++t) {
+    __syncthreads();
+    for (int i = threadIdx.x; i < KD; i += blockDim.x) {
+      ks[i] = i < dim ? kn[((int64_t)t * kv_heads + hk) * dim + i] : 0.f;
+      qs[i] = i < dim ? qn[((int64_t)t * kv_heads + hk) * dim + i] : 0.f;
+    }
+    __syncthreads();
+    const float gt = g[(int64_t)t * heads + h], bt = beta[(int64_t)t * heads + h];
+    const float vt = active ? Elem<T>::load(qkv[(int64_t)t * qkv_stride + v_offset + h * vdim + j]) : 0.f;
+    float dot = 0.f;
+#pragma unroll
+    for (int i = 0; i < KD; ++i) {
+      S[i] *= gt;
+      dot += S[i] * ks[i];
+    }
+    const float u = bt * (vt - dot);
+    float o = 0.f;
+#pragma unroll
+    for (int i = 0; i < KD; ++i) {
+      S[i] += ks[i] * u;
+      o += S[i] * qs[i];
+    }
+    if (active) out[((int64_t)t * heads + h) * vdim + j] = o;
+  }
+  if (active) {
+#pragma unroll
+    for (int i = 0; i < KD; ++i)
+      if (i < dim) held[(int64_t)i * vdim + j] = S[i];
+  }
+}
+
+// Per (row, head): o = (S + diag(u) k v^T)^T r; S <- diag(w) S + k v^T. Thread j owns column j of S [D, D].
+template <int KD, typename T>
+__global__ void __launch_bounds__(WAVE) memory_scan_kernel(const T* __restrict__ r, const T* __restrict__ k, const T* __restrict__ v,
+                                   const float* __restrict__ w, const float* __restrict__ u, float* __restrict__ state,
+                                   float* __restrict__ out, const int32_t* __restrict__ slots,
+                                   const int32_t* __restrict__ starts, const int32_t* __restrict__ query_start,
+                                   int heads, int dim) {
+  __shared__ float rs[KD], ks[KD], ws[KD], us[KD];
+  const int b = blockIdx.x, h = blockIdx.y, j = blockIdx.z * WAVE + threadIdx.x;
+  const bool active = j < dim;
+  const int lo = query_start[b], hi = query_start[b + 1];
+  float* held = state + ((int64_t)slots[b] * heads + h) * dim * dim;
+  const bool carried = starts[b] > 0;
+  float S[KD];
+#pragma unroll
+  for (int i = 0; i < KD; ++i) S[i] = (carried && active && i < dim) ? held[(int64_t)i * dim + j] : 0.f;
+  for (int i = threadIdx.x; i < KD; i += blockDim.x) us[i] = i < dim ? u[h * dim + i] : 0.f;
+  const int64_t width = (int64_t)heads * dim;
+  for (int t = lo; t < hi; ++t) {
+    __syncthreads();
+    for (int i = threadIdx.x; i < KD; i += blockDim.x) {
+      const int64_t at = (int64_t)t * width + h * dim + i;
+      rs[i] = i < dim ? Elem<T>::load(r[at]) : 0.f;
+      ks[i] = i < dim ? Elem<T>::load(k[at]) : 0.f;
+      ws[i] = i < dim ? w[at] : 0.f;
+    }
+    __syncthreads();
+    const float vt = active ? Elem<T>::load(v[(int64_t)t * width + h * dim + j]) : 0.f;
+    float o = 0.f;
+#pragma unroll
+    for (int i = 0; i < KD; ++i) {
+      const float kv = ks[i] * vt;
+      o += rs[i] * (S[i] + us[i] * kv);
+      S[i] = ws[i] * S[i] + kv;
+    }
+    if (active) out[(int64_t)t * width + h * dim + j] = o;
+  }
+  if (active) {
+#pragma unroll
+    for (int i = 0; i < KD; ++i)
+      if (i < dim) held[(int64_t)i * dim + j] = S[i];
+  }
+}
+
+// One wave per (token, head): o / sqrt(mean(o^2) + eps) * weight * silu(gate).
+template <typename T>
+__global__ void __launch_bounds__(256) gated_out_kernel(const float* __restrict__ o, const T* __restrict__ gate,
+                                                        const T* __restrict__ weight, T* __restrict__ y, int64_t cells,
+                                                        int heads, int vdim, int per_head, float eps) {
+  const int64_t cell = (int64_t)blockIdx.x * 4 + threadIdx.x / WAVE;
+  const int lane = threadIdx.x % WAVE;
+  if (cell >= cells) return;
+  const int h = (int)(cell % heads);
+  const float* src = o + cell * vdim;
+  float ss = 0.f;
+  for (int d = lane; d < vdim; d += WAVE) ss += src[d] * src[d];
+  ss = wave_sum(ss);
+  const float r = 1.0f / sqrtf(ss / (float)vdim + eps);
+  for (int d = lane; d < vdim; d += WAVE) {
+    const float wv = Elem<T>::load(weight[per_head ? h * vdim + d : d]);
+    const float gv = Elem<T>::load(gate[cell * vdim + d]);
+    y[cell * vdim + d] = Elem<T>::store(src[d] * r * wv * silu<T>(gv));
+  }
+}
+
+template <typename T>
+__global__ void shift_mix_kernel(const T* __restrict__ x, const T* __restrict__ mu, const T* __restrict__ state,
+                                 T* __restrict__ y, const int32_t* __restrict__ slots, const int32_t* __restrict__ starts,
+                                 const int32_t* __restrict__ query_start, const int32_t* __restrict__ token_row,
+                                 int tokens, int width, int mixes) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  const int t = blockIdx.y;
+  if (c >= width) return;
+  const int b = token_row[t];
+  float prev = 0.f;
+  if (t > query_start[b]) prev = Elem<T>::load(x[(int64_t)(t - 1) * width + c]);
+  else if (starts[b] > 0) prev = Elem<T>::load(state[(int64_t)slots[b] * width + c]);
+  const float cur = Elem<T>::load(x[(int64_t)t * width + c]);
+  for (int s = 0; s < mixes; ++s)
+    y[((int64_t)s * tokens + t) * width + c] = Elem<T>::store(cur + (prev - cur) * Elem<T>::load(mu[(int64_t)s * width + c]));
+}
+
+template <typename T>
+__global__ void shift_keep_kernel(const T* __restrict__ x, T* __restrict__ state, const int32_t* __restrict__ slots,
+                                  const int32_t* __restrict__ query_start, int width) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  const int b = blockIdx.y;
+  if (c >= width) return;
+  state[(int64_t)slots[b] * width + c] = x[(int64_t)(query_start[b + 1] - 1) * width + c];
+}
+
+// One block a token: exp(-exp(tanh(a) w2^T + w0)), the rank's tanh values shared through LDS.
+template <typename T>
+__global__ void __launch_bounds__(256) decay_lora_kernel(const float* __restrict__ a, const T* __restrict__ w2,
+                                                         const float* __restrict__ w0, float* __restrict__ y,
+                                                         int channels, int rank) {
+  __shared__ float th[1024];
+  const int t = blockIdx.x;
+  for (int r = threadIdx.x; r < rank; r += 256) th[r] = tanhf(a[(int64_t)t * rank + r]);
+  __syncthreads();
+  for (int c = threadIdx.x; c < channels; c += 256) {
+    float acc = 0.f;
+    for (int r = 0; r < rank; ++r) acc += th[r] * Elem<T>::load(w2[(int64_t)c * rank + r]);
+    y[(int64_t)t * channels + c] = expf(-expf(acc + w0[c]));
+  }
+}
+
+}  // namespace
+
+#define BY_DTYPE(dtype, CALL)                    \
+  do {                                           \
+    if ((dtype) == HOLON_F32) { using T = float; CALL; } \
+    else { using T = bf16_t; CALL; }             \
+  } while (0)
+
+extern "C" int holon_causal_conv(const void* x, const void* w, void* state, void* y, const int32_t* slots,
+                                 const int32_t* starts, const int32_t* query_start, const int32_t* token_row,
+                                 int tokens, int rows, int channels, int taps, int state_slots, int add_input, int act,
+                                 int dtype, void* stream) {
+  HOLON_CHECK(tokens >= 0 && rows >= 0 && channels > 0 && taps >= 1 && taps <= 16 && state_slots > 0,
+              "causal_conv: tokens=%d rows=%d channels=%d taps=%d", tokens, rows, channels, taps);
+  HOLON_CHECK(tokens <= 65535 && rows <= 65535, "causal_conv: %d tokens in %d rows exceed one launch", tokens, rows);
+  if (tokens == 0 || rows == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 block(256), grid_t((channels + 255) / 256, tokens), grid_b((channels + 255) / 256, rows);
+  BY_DTYPE(dtype, (causal_conv_kernel<T><<<grid_t, block, 0, s>>>((const T*)x, (const T*)w, (const T*)state, (T*)y, slots,
+                                                                  starts, query_start, token_row, channels, taps,
+                                                                  add_input, act)));
+  HOLON_LAUNCH_OK();
+  if (taps > 1) {
+    BY_DTYPE(dtype, (causal_conv_keep_kernel<T><<<grid_b, block, 0, s>>>((const T*)x, (T*)state, slots, starts,
+                                                                         query_start, channels, taps)));
+    HOLON_LAUNCH_OK();
+  }
+  return 0;
+}
+
+extern "C" int holon_delta_prepare(const void* qkv, const void* ab, const float* a_log, const float* dt_bias, float* qn,
+                                   float* kn, float* beta, float* g, int tokens, int heads, int kv_heads, int dim,
+                                   int vdim, int dtype, void* stream) {
+  HOLON_CHECK(tokens >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dim > 0 && vdim > 0,
+              "delta_prepare: %d/%d heads of %d/%d", heads, kv_heads, dim, vdim);
+  if (tokens == 0) return 0;
+  BY_DTYPE(dtype, (delta_prepare_kernel<T><<<tokens, 256, 0, (hipStream_t)stream>>>(
+                      (const T*)qkv, (const T*)ab, a_log, dt_bias, qn, kn, beta, g, heads, kv_heads, dim, vdim)));
+  HOLON_LAUNCH_OK();
+  return 0;
+}
+
+template <typename T, int KD>
+static void launch_delta(dim3 grid, hipStream_t s, const float* qn, const float* kn, const void* qkv,
+                         int stride, int voff, const float* beta, const float* g, float* state, float* out,
+                         const int32_t* slots, const int32_t* starts, const int32_t* qs, int heads, int kv_heads, int dim,
+                         int vdim) {
+  delta_scan_kernel<KD, T><<<grid, WAVE, 0, s>>>(qn, kn, (const T*)qkv, stride, voff, beta, g, state, out, slots,
+                                                    starts, qs, heads, kv_heads, dim, vdim);
+}
+
+#define BY_KEY_SIZE(dim, CALL)                                  \
+  do {                                                          \
+    if ((dim) <= 16) { constexpr int KD = 16; CALL; }           \
+    else if ((dim) <= 32) { constexpr int KD = 32; CALL; }      \
+    else if ((dim) <= 48) { constexpr int KD = 48; CALL; }      \
+    else if ((dim) <= 64) { constexpr int KD = 64; CALL; }      \
+    else if ((dim) <= 96) { constexpr int KD = 96; CALL; }      \
+    else if ((dim) <= 128) { constexpr int KD = 128; CALL; }    \
+    else if ((dim) <= 192) { constexpr int KD = 192; CALL; }    \
+    else { constexpr int KD = 256; CALL; }                      \
+  } while (0)
+
+extern "C" int holon_delta_scan(const float* qn, const float* kn, const void* qkv, int qkv_stride, int v_offset,
+                                const float* beta, const float* g, float* state, float* out, const int32_t* slots,
+                                const int32_t* starts, const int32_t* query_start, int rows, int heads, int kv_heads,
+                                int dim, int vdim, int state_slots, int dtype, void* stream) {
+  HOLON_CHECK(rows >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "delta_scan: %d/%d heads", heads, kv_heads);
+  HOLON_CHECK(dim > 0 && dim <= 256 && vdim > 0 && vdim <= 1024, "delta_scan: key size %d (at most 256), value size %d "
+              "(at most 1024)", dim, vdim);
+  HOLON_CHECK(rows <= 0x7fffffff / 2 && heads <= 65535 && state_slots > 0 && v_offset >= 0 &&
+              v_offset + heads * vdim <= qkv_stride, "delta_scan: launch or row layout out of range");
+  if (rows == 0) return 0;
+  const dim3 grid(rows, heads, (vdim + WAVE - 1) / WAVE);     // a wave for every 64 value columns
+  hipStream_t s = (hipStream_t)stream;
+  BY_DTYPE(dtype, BY_KEY_SIZE(dim, (launch_delta<T, KD>(grid, s, qn, kn, qkv, qkv_stride, v_offset, beta, g,
+                                                         state, out, slots, starts, query_start, heads, kv_heads, dim,
+                                                         vdim))));
+  HOLON_LAUNCH_OK();
+  return 0;
+}
+
+template <typename T, int KD>
+static void launch_memory(dim3 grid, hipStream_t s, const void* r, const void* k, const void* v,
+                          const float* w, const float* u, float* state, float* out, const int32_t* slots,
+                          const int32_t* starts, const int32_t* qs, int heads, int dim) {
+  memory_scan_kernel<KD, T><<<grid, WAVE, 0, s>>>((const T*)r, (const T*)k, (const T*)v, w, u, state, out, slots,
+                                                     starts, qs, heads, dim);
+}
+
+extern "C" int holon_memory_scan(const void* r, const void* k, const void* v, const float* w, const float* u,
+                                 float* state, float* out, const int32_t* slots, const int32_t* starts,
+                                 const int32_t* query_start, int rows, int heads, int dim, int state_slots, int dtype,
+                                 void* stream) {
+  HOLON_CHECK(rows >= 0 && heads > 0 && heads <= 65535 && dim > 0 && dim <= 256 && state_slots > 0,
+              "memory_scan: %d heads of %d (at most 256)", heads, dim);
+  if (rows == 0) return 0;
+  const dim3 grid(rows, heads, (dim + WAVE - 1) / WAVE);
+  hipStream_t s = (hipStream_t)stream;
+  BY_DTYPE(dtype, BY_KEY_SIZE(dim, (launch_memory<T, KD>(grid, s, r, k, v, w, u, state, out, slots, starts,
+                                                          query_start, heads, dim))));
+  HOLON_LAUNCH_OK();
+  return 0;
+}
+
+extern "C" int holon_gated_out(const float* o, const void* gate, const void* weight, void* y, int tokens, int heads,
+                               int vdim, int per_head, float eps, int dtype, void* stream) {
+  HOLON_CHECK(tokens >= 0 && heads > 0 && vdim > 0, "gated_out: %d heads of %d", heads, vdim);
+  const int64_t cells = (int64_t)tokens * heads;
+  if (cells == 0) return 0;
+  HOLON_CHECK((cells + 3) / 4 <= 0x7fffffff, "gated_out: %lld cells exceed one launch", (long long)cells);
+  BY_DTYPE(dtype, (gated_out_kernel<T><<<(unsigned)((cells + 3) / 4), 256, 0, (hipStream_t)stream>>>(
+                      o, (const T*)gate, (const T*)weight, (T*)y, cells, heads, vdim, per_head, eps)));
+  HOLON_LAUNCH_OK();
+  return 0;
+}
+
+extern "C" int holon_shift_mix(const void* x, const void* mu, void* state, void* y, const int32_t* slots,
+                               const int32_t* starts, const int32_t* query_start, const int32_t* token_row, int tokens,
+                               int rows, int width, int mixes, int state_slots, int dtype, void* stream) {
+  HOLON_CHECK(tokens >= 0 && rows >= 0 && width > 0 && mixes > 0 && state_slots > 0, "shift_mix: tokens=%d width=%d",
+              tokens, width);
+  HOLON_CHECK(tokens <= 65535 && rows <= 65535, "shift_mix: %d tokens in %d rows exceed one launch", tokens, rows);
+  if (tokens == 0 || rows == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 block(256), grid_t((width + 255) / 256, tokens), grid_b((width + 255) / 256, rows);
+  BY_DTYPE(dtype, (shift_mix_kernel<T><<<grid_t, block, 0, s>>>((const T*)x, (const T*)mu, (const T*)state, (T*)y, slots,
+                                                                starts, query_start, token_row, tokens, width, mixes)));
+  HOLON_LAUNCH_OK();
+  BY_DTYPE(dtype, (shift_keep_kernel<T><<<grid_b, block, 0, s>>>((const T*)x, (T*)state, slots, query_start, width)));
+  HOLON_LAUNCH_OK();
+  return 0;
+}
+
+extern "C" int holon_decay_lora(const float* a, const void* w2, const float* w0, float* y, int tokens, int channels,
+                                int rank, int dtype, void* stream) {
+  HOLON_CHECK(tokens >= 0 && channels > 0 && rank > 0 && rank <= 1024, "decay_lora: %d channels, rank %d (at most 1024)",
+              channels, rank);
+  if (tokens == 0) return 0;
+  BY_DTYPE(dtype, (decay_lora_kernel<T><<<tokens, 256, 0, (hipStream_t)stream>>>(a, (const T*)w2, w0, y, channels, rank)));
+  HOLON_LAUNCH_OK();
+  return 0;
+}

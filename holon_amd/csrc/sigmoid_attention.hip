@@ -1,0 +1,212 @@
+// Windowed attention with sigmoid weights over a paged cache whose keys and values may differ in width.
+//
+// One page of one site holds P tokens: keys [Hkv, P, D] followed by values [Hkv, P, V], token-major. `head_prepare`
+// norms and rotates the heads of a merged q/k/v projection and stores keys and values; `sigmoid_attention` sums
+// sigmoid(q . k * scale + bias) * v over the keys a query sees. Nothing is normalised over keys, so there is no running
+// maximum and no rescaling: a query's result is a plain sum, taken over its keys from the oldest visible one on, in
+// tiles of 64, an order that the query's position alone decides. Scores, weights and sums are float32.
+#include "common.h"
+#include "holon_hip.h"
+
+#define SIG_MAX_D 512
+
+namespace {
+
+// One wave per (token, head of q, k or v). q and k: x * rsqrt(mean(x^2) + eps) * weight (if weights), then the
+// half-split rotation of the first `rot` dimensions; one rounding.
+template <typename T>
+__global__ void __launch_bounds__(256) head_prepare_kernel(const T* __restrict__ qkv, T* __restrict__ q_out, int heads,
+                                                           int kv_heads, int dim, int vdim,
+                                                           const T* __restrict__ q_weight, const T* __restrict__ k_weight,
+                                                           float eps, const float* __restrict__ table, int rot,
+                                                           int table_rows, const int32_t* __restrict__ positions,
+                                                           T* __restrict__ pages, const int32_t* __restrict__ write_page,
+                                                           const int32_t* __restrict__ write_off, int page_size,
+                                                           int num_pages) {
+  const int t = blockIdx.x;
+  const int hs = blockIdx.y * 4 + threadIdx.x / WAVE;
+  const int lane = threadIdx.x % WAVE;
+  if (hs >= heads + 2 * kv_heads) return;
+  const int64_t width = (int64_t)(heads + kv_heads) * dim + (int64_t)kv_heads * vdim;
+  const int64_t page_len = (int64_t)kv_heads * page_size * (dim + vdim);
+  const T* row = qkv + (int64_t)t * width;
+  const int page = write_page[t], off = write_off[t];
+  const bool page_ok = page >= 0 && page < num_pages && off >= 0 && off < page_size;
+  if (hs >= heads + kv_heads) {                       // a value head: stored as it is
+    const int hv = hs - heads - kv_heads;
+    if (!page_ok) return;
+    const T* src = row + (int64_t)(heads + kv_heads) * dim + (int64_t)hv * vdim;
+    T* dst = pages + page * page_len + (int64_t)kv_heads * page_size * dim + ((int64_t)hv * page_size + off) * vdim;
+    for (int d = lane; d < vdim; d += WAVE) dst[d] = src[d];
+    return;
+  }
+  const bool is_q = hs < heads;
+  if (!is_q && !page_ok) return;
+  const T* src = row + (int64_t)hs * dim;
+  T* dst = is_q ? q_out + ((int64_t)t * heads + hs) * dim
+                : pages + page * page_len + ((int64_t)(hs - heads) * page_size + off) * dim;
+  const T* w = is_q ? q_weight : k_weight;
+  float r = 1.f;
+  if (w) {
+    float ss = 0.f;
+    for (int d = lane; d < dim; d += WAVE) {
+      const float v = Elem<T>::load(src[d]);
+      ss += v * v;
+    }
+    r = 1.0f / sqrtf(wave_sum(ss) / (float)dim + eps);
+  }
+  const int half = rot / 2;
+  if (table) {
+    int pos = positions[t];
+    pos = pos < 0 ? 0 : (pos >= table_rows ? table_rows - 1 : pos);
+    const float* cs = table + (int64_t)pos * rot;
+    for (int p = lane; p < half; p += WAVE) {
+      const float a = Elem<T>::load(src[p]) * r * (w ? Elem<T>::load(w[p]) : 1.f);
+      const float b = Elem<T>::load(src[p + half]) * r * (w ? Elem<T>::load(w[p + half]) : 1.f);
+      const float c = cs[p], s = cs[half + p];
+      dst[p] = Elem<T>::store(a * c - b * s);
+      dst[p + half] = Elem<T>::store(b * c + a * s);
+    }
+  }
+  for (int d = (table ? rot : 0) + lane; d < dim; d += WAVE)
+    dst[d] = Elem<T>::store(Elem<T>::load(src[d]) * r * (w ? Elem<T>::load(w[d]) : 1.f));
+}
+
+// One wave per (token, head), four heads of a token per block. A lane takes one key of a tile of 64: its score over D
+// (the query comes from LDS), its weight; then the lanes turn to the value columns and add the tile's weighted values.
+template <typename T, bool VEC>
+__global__ void __launch_bounds__(256) sigmoid_attention_kernel(const T* __restrict__ q, T* __restrict__ out,
+                                                                const T* __restrict__ pages,
+                                                                const int32_t* __restrict__ table, int table_stride,
+                                                                const int32_t* __restrict__ slots,
+                                                                const int32_t* __restrict__ token_row,
+                                                                const int32_t* __restrict__ positions, int heads,
+                                                                int kv_heads, int dim, int vdim, int page_size,
+                                                                const float* __restrict__ bias, float scale, int window,
+                                                                const T* __restrict__ gate) {
+  __shared__ float q_s[4][SIG_MAX_D];
+  __shared__ float p_s[4][WAVE];
+  __shared__ int64_t v_s[4][WAVE];
+  const int w = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  const int t = blockIdx.x;
+  const bool live = blockIdx.y * 4 + w < heads;
+  const int h = live ? blockIdx.y * 4 + w : 0;       // a spare wave walks head 0 and stores nothing: all reach the barriers
+  const int pos = positions[t];
+  const int hk = h / (heads / kv_heads);
+  const int32_t* trow = table + (int64_t)slots[token_row[t]] * table_stride;
+  const int64_t page_len = (int64_t)kv_heads * page_size * (dim + vdim);
+  const int64_t val_base = (int64_t)kv_heads * page_size * dim;
+  const T* qp = q + ((int64_t)t * heads + h) * dim;
+  for (int d = lane; d < dim; d += WAVE) q_s[w][d] = Elem<T>::load(qp[d]);
+  __syncthreads();
+  const float head_bias = bias ? bias[h] : 0.f;
+  const int first = window > 0 ? max(0, pos - window + 1) : 0;
+  float acc[SIG_MAX_D / WAVE];
+#pragma unroll
+  for (int i = 0; i < SIG_MAX_D / WAVE; ++i) acc[i] = 0.f;
+  constexpr int V = Elem<T>::kVec;
+
+  for (int j0 = first; j0 <= pos; j0 += WAVE) {
+    const int key = j0 + lane;
+    float p = 0.f;
+    int64_t voff = 0;
+    if (key <= pos) {
+      const int page = trow[key / page_size];
+      const int off = key - (key / page_size) * page_size;
+      const T* kp = pages + page * page_len + ((int64_t)hk * page_size + off) * dim;
+      voff = page * page_len + val_base + ((int64_t)hk * page_size + off) * vdim;
+      float dot = 0.f;
+      if (VEC) {
+        for (int d = 0; d < dim; d += V) {
+          const uint4 raw = *reinterpret_cast<const uint4*>(kp + d);
+          const T* e = reinterpret_cast<const T*>(&raw);
+#pragma unroll
+          for (int i = 0; i < V; ++i) dot += q_s[w][d + i] * Elem<T>::load(e[i]);
+        }
+      } else {
+        for (int d = 0; d < dim; ++d) dot += q_s[w][d] * Elem<T>::load(kp[d]);
+      }
+      p = 1.0f / (1.0f + expf(-(dot * scale + head_bias)));
+    }
+    p_s[w][lane] = p;
+    v_s[w][lane] = voff;
+    __syncthreads();
+    const int count = min(WAVE, pos - j0 + 1);
+#pragma unroll
+    for (int i = 0; i < SIG_MAX_D / WAVE; ++i) {
+      const int d = lane + i * WAVE;
+      if (d < vdim) {
+        float a = acc[i];
+        for (int j = 0; j < count; ++j) a += p_s[w][j] * Elem<T>::load(pages[v_s[w][j] + d]);
+        acc[i] = a;
+      }
+    }
+    __syncthreads();
+  }
+  if (!live) return;
+#pragma unroll
+  for (int i = 0; i < SIG_MAX_D / WAVE; ++i) {
+    const int d = lane + i * WAVE;
+    if (d < vdim) {
+      const int64_t at = ((int64_t)t * heads + h) * vdim + d;
+      float o = acc[i];
+      if (gate) o *= 1.0f / (1.0f + expf(-Elem<T>::load(gate[at])));
+      out[at] = Elem<T>::store(o);
+    }
+  }
+}
+}  // namespace
+
+extern "C" int holon_head_prepare(const void* qkv, void* q_out, int tokens, int heads, int kv_heads, int dim, int vdim,
+                                  const void* q_weight, const void* k_weight, float eps, const float* table, int rot,
+                                  int table_rows, const int32_t* positions, void* pages, const int32_t* write_page,
+                                  const int32_t* write_off, int page_size, int num_pages, int dtype, void* stream) {
+  HOLON_CHECK(tokens >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dim > 0 && vdim > 0,
+              "head_prepare: %d/%d heads of %d/%d", heads, kv_heads, dim, vdim);
+  HOLON_CHECK((table == nullptr && rot == 0) || (rot > 0 && rot % 2 == 0 && rot <= dim && table_rows > 0),
+              "head_prepare: %d rotary dimensions for heads of %d", rot, dim);
+  HOLON_CHECK(page_size > 0 && num_pages > 0 && (q_weight == nullptr) == (k_weight == nullptr),
+              "head_prepare: bad page geometry or one norm weight without the other");
+  if (tokens == 0) return 0;
+  HOLON_CHECK((heads + 2 * kv_heads + 3) / 4 <= 65535, "head_prepare: too many heads for one launch");
+  const dim3 grid(tokens, (heads + 2 * kv_heads + 3) / 4);
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == HOLON_F32)
+    head_prepare_kernel<float><<<grid, 256, 0, s>>>((const float*)qkv, (float*)q_out, heads, kv_heads, dim, vdim,
+                                                    (const float*)q_weight, (const float*)k_weight, eps, table, rot,
+                                                    table_rows, positions, (float*)pages, write_page, write_off,
+                                                    page_size, num_pages);
+  else
+    head_prepare_kernel<bf16_t><<<grid, 256, 0, s>>>((const bf16_t*)qkv, (bf16_t*)q_out, heads, kv_heads, dim, vdim,
+                                                     (const bf16_t*)q_weight, (const bf16_t*)k_weight, eps, table, rot,
+                                                     table_rows, positions, (bf16_t*)pages, write_page, write_off,
+                                                     page_size, num_pages);
+  HOLON_LAUNCH_OK();
+  return 0;
+}
+
+extern "C" int holon_sigmoid_attention(const void* q, void* out, const void* pages, const int32_t* table,
+                                       int table_stride, const int32_t* slots, const int32_t* token_row,
+                                       const int32_t* positions, int tokens, int heads, int kv_heads, int dim, int vdim,
+                                       int page_size, int num_pages, const float* bias, float scale, int window,
+                                       const void* gate, int dtype, void* stream) {
+  HOLON_CHECK(tokens >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "sigmoid_attention: %d/%d heads", heads,
+              kv_heads);
+  HOLON_CHECK(dim > 0 && dim <= SIG_MAX_D && vdim > 0 && vdim <= SIG_MAX_D,
+              "sigmoid_attention: head sizes %d/%d (at most %d)", dim, vdim, SIG_MAX_D);
+  HOLON_CHECK(page_size > 0 && num_pages > 0 && window >= 0 && table_stride > 0, "sigmoid_attention: bad page geometry");
+  if (tokens == 0) return 0;
+  const dim3 grid(tokens, (heads + 3) / 4);
+  hipStream_t s = (hipStream_t)stream;
+  const int vec = dtype == HOLON_F32 ? 4 : 8;
+  const bool aligned = dim % vec == 0 && vdim % vec == 0 && (uintptr_t)pages % 16 == 0;
+#define SIG_LAUNCH(T, VEC)                                                                                            \
+  sigmoid_attention_kernel<T, VEC><<<grid, 256, 0, s>>>((const T*)q, (T*)out, (const T*)pages, table, table_stride,  \
+                                                        slots, token_row, positions, heads, kv_heads, dim, vdim,     \
+                                                        page_size, bias, scale, window, (const T*)gate)
+  if (dtype == HOLON_F32) { if (aligned) SIG_LAUNCH(float, true); else SIG_LAUNCH(float, false); }
+  else { if (aligned) SIG_LAUNCH(bf16_t, true); else SIG_LAUNCH(bf16_t, false); }
+#undef SIG_LAUNCH
+  HOLON_LAUNCH_OK();
+  return 0;
+}

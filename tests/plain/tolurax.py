@@ -99,12 +99,11 @@ def windowed_sigmoid_attention(h, p, m, eps, get):
     size = m["mask"]["size"]
     bias = get(p + "pb")
     out = torch.zeros(T, H, V, dtype=h.dtype)
+    k, v = k.repeat_interleave(H // G, dim=1), v.repeat_interleave(H // G, dim=1)     # head hd reads kv head hd // (H/G)
     for t in range(T):
-        for hd in range(H):
-            kv = hd // (H // G)
-            for s in range(max(0, t - size + 1), t + 1):
-                score = (q[t, hd] * k[s, kv]).sum() * m["scale"]
-                out[t, hd] += sigmoid(score + bias[hd]) * v[s, kv]
+        first = max(0, t - size + 1)
+        score = torch.einsum("hd,shd->sh", q[t], k[first: t + 1]) * m["scale"]     # [visible keys, H]
+        out[t] = torch.einsum("sh,shv->hv", sigmoid(score + bias), v[first: t + 1])
     gate = sigmoid(h @ get(p + "g").T)
     return (out.reshape(T, H * V) * gate) @ get(p + "o").T
 
@@ -127,10 +126,9 @@ def decayed_outer_memory(h, p, m, eps, get):
     S = torch.zeros(H, D, D, dtype=h.dtype)
     out = torch.zeros(T, H, D, dtype=h.dtype)
     for t in range(T):
-        for hd in range(H):
-            kv = torch.outer(k[t, hd], v[t, hd])
-            out[t, hd] = (S[hd] + u[hd][:, None] * kv).T @ r[t, hd]
-            S[hd] = decay[t, hd][:, None] * S[hd] + kv
+        kv = k[t][:, :, None] * v[t][:, None, :]                           # [H, D, D]: k v^T per head
+        out[t] = torch.einsum("hdv,hd->hv", S + u[:, :, None] * kv, r[t])
+        S = decay[t][:, :, None] * S + kv
     out = rms_div(out, eps).reshape(T, H * D) * get(p + "norm") * gate
     return out @ get(p + "o").T
 
@@ -149,13 +147,12 @@ def gated_delta(h, p, m, eps, get):
     g = torch.exp(-torch.exp(get(p + "A_log")) * softplus(h @ get(p + "a").T + get(p + "dt_bias")))
     S = torch.zeros(H, D, V, dtype=h.dtype)
     out = torch.zeros(T, H, V, dtype=h.dtype)
+    q, k = q.repeat_interleave(H // G, dim=1), k.repeat_interleave(H // G, dim=1)     # head hd reads q/k head hd // (H/G)
     for t in range(T):
-        for hd in range(H):
-            kv = hd // (H // G)
-            S[hd] = g[t, hd] * S[hd]
-            u = beta[t, hd] * (v[t, hd] - S[hd].T @ k[t, kv])
-            S[hd] = S[hd] + torch.outer(k[t, kv], u)
-            out[t, hd] = S[hd].T @ q[t, kv]
+        S = g[t][:, None, None] * S
+        u = beta[t][:, None] * (v[t] - torch.einsum("hdv,hd->hv", S, k[t]))
+        S = S + k[t][:, :, None] * u[:, None, :]
+        out[t] = torch.einsum("hdv,hd->hv", S, q[t])
     out = rms_div(out, eps) * get(p + "norm")
     return (out.reshape(T, H * V) * silu(h @ get(p + "g").T)) @ get(p + "o").T
 
