@@ -188,7 +188,8 @@ def forward(config, tensors, tokens, dtype=torch.float64):
         if pass_start:
             x = torch.cat((x, x0), dim=-1) @ get("loop.in").T
         h = layer_norm(x, get(p + "norm1"), eps)
-        h = h + causal_conv(h, get(p + "canon1"))
+        if config.get("canon"):
+            h = h + causal_conv(h, get(p + "canon1"))
         m = layer["mixer"]
         if layer["type"] == "delta":
             y = gated_delta(h, p + "mix.", m, eps, get)
