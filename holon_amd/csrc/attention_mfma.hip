@@ -57,6 +57,11 @@ struct AttnArgs {
   int rows_in_order;       // every row of the step is a decode row and row_ids[i] = query_start[i] = i
   // long prompt portions only: a block runs one of its two ranges (blockIdx.z = 2 row + which), not both
   int unpaired;
+  // sigmoid weights instead of a softmax (the wide prompt kernel only): p = 1 / (1 + exp(-(s * scale + head_bias[head]))),
+  // nothing normalised; `gate` (nullable, [T, Hq D]): the result is multiplied by its sigmoid
+  float scale;
+  const float* head_bias;
+  const bf16_t* gate;
 };
 
 // How the 16 rows of a tile map to (position, head) for a group of G heads.
@@ -572,7 +577,9 @@ __host__ __device__ inline TileMap32 tile_map32(int group) {
   return m;
 }
 
-template <int D>
+// SIG: sigmoid weights (see AttnArgs). A weight is then split into its bfloat16 rounding and the rounding of what is
+// left, and the value product runs over both: the weights enter the sum with 16 bits of mantissa, not 8.
+template <int D, bool SIG = false>
 __global__ void __launch_bounds__(256, D == 128 ? 2 : 3) attn_prefill_wide_kernel(AttnArgs a) {
   constexpr int KP = D + 8;    // pitch of a key row in LDS (elements)
   constexpr int VP = 40;       // pitch of a value row: 32 keys + 8
@@ -658,6 +665,7 @@ __global__ void __launch_bounds__(256, D == 128 ? 2 : 3) attn_prefill_wide_kerne
 #pragma unroll
       for (int i = 0; i < 16; ++i) o[db][i] = 0.f;
     float m = -INFINITY, l = 0.f;
+    const float sig_bias = SIG && valid && a.head_bias ? a.head_bias[head] : 0.f;
 
     struct Regs { bf16x8_t k[ROUNDS], v[ROUNDS]; };
     Regs r0, r1;
@@ -724,6 +732,24 @@ __global__ void __launch_bounds__(256, D == 128 ? 2 : 3) attn_prefill_wide_kerne
             if (!(key <= qpos && key >= first)) sv[idx] = -INFINITY;
           }
         }
+        if constexpr (SIG) {
+          bf16x8_t pb0, pb1, pl0, pl1;
+#pragma unroll
+          for (int idx = 0; idx < 16; ++idx) {       // (a masked score is -inf)
+            const float e = __builtin_amdgcn_exp2f(-(fmaf(sv[idx], a.scale, sig_bias)) * 1.4426950408889634f);
+            const float p = sv[idx] == -INFINITY ? 0.f : __builtin_amdgcn_rcpf(1.0f + e);
+            const __bf16 hi = (__bf16)p;
+            const __bf16 lo = (__bf16)(p - (float)hi);
+            if (idx < 8) { pb0[idx] = hi; pl0[idx] = lo; } else { pb1[idx - 8] = hi; pl1[idx - 8] = lo; }
+          }
+#pragma unroll
+          for (int db = 0; db < D / 32; ++db) {
+            o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[db][0], pb0, o[db], 0, 0, 0);
+            o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[db][0], pl0, o[db], 0, 0, 0);
+            o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[db][1], pb1, o[db], 0, 0, 0);
+            o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[db][1], pl1, o[db], 0, 0, 0);
+          }
+        } else {
         float mx = sv[0];
 #pragma unroll
         for (int idx = 1; idx < 16; ++idx) mx = fmaxf(mx, sv[idx]);
@@ -754,6 +780,7 @@ __global__ void __launch_bounds__(256, D == 128 ? 2 : 3) attn_prefill_wide_kerne
           o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[db][0], pb0, o[db], 0, 0, 0);
           o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[db][1], pb1, o[db], 0, 0, 0);
         }
+        }
       }
       if constexpr (!decltype(last)::value) {
         stash(buf ^ 1, next);
@@ -781,17 +808,26 @@ __global__ void __launch_bounds__(256, D == 128 ? 2 : 3) attn_prefill_wide_kerne
     }
     float lt = l + __shfl_xor(l, 32, WAVE);
     if (valid) {
-      const float inv = lt > 0.f ? 1.0f / lt : 0.f;
+      const float inv = SIG ? 1.0f : (lt > 0.f ? 1.0f / lt : 0.f);
       bf16_t* op = a.out + ((int64_t)token * a.heads + head) * D + 4 * h;
+      const bf16_t* gp = SIG && a.gate ? a.gate + ((int64_t)token * a.heads + head) * D + 4 * h : nullptr;
 #pragma unroll
       for (int db = 0; db < D / 32; ++db)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
+          float gs[4] = {1.f, 1.f, 1.f, 1.f};
+          if (SIG && gp) {
+            const ushort4 gv = *reinterpret_cast<const ushort4*>(gp + db * 32 + 8 * i);
+            gs[0] = 1.0f / (1.0f + __expf(-bf16_to_float(gv.x)));
+            gs[1] = 1.0f / (1.0f + __expf(-bf16_to_float(gv.y)));
+            gs[2] = 1.0f / (1.0f + __expf(-bf16_to_float(gv.z)));
+            gs[3] = 1.0f / (1.0f + __expf(-bf16_to_float(gv.w)));
+          }
           ushort4 w;
-          w.x = float_to_bf16(o[db][4 * i + 0] * inv);
-          w.y = float_to_bf16(o[db][4 * i + 1] * inv);
-          w.z = float_to_bf16(o[db][4 * i + 2] * inv);
-          w.w = float_to_bf16(o[db][4 * i + 3] * inv);
+          w.x = float_to_bf16(o[db][4 * i + 0] * inv * gs[0]);
+          w.y = float_to_bf16(o[db][4 * i + 1] * inv * gs[1]);
+          w.z = float_to_bf16(o[db][4 * i + 2] * inv * gs[2]);
+          w.w = float_to_bf16(o[db][4 * i + 3] * inv * gs[3]);
           *reinterpret_cast<ushort4*>(op + db * 32 + 8 * i) = w;
         }
     }
@@ -1769,6 +1805,36 @@ extern "C" int holon_attention_prefill_bf16(const void* q, void* out, const void
   if (head_dim == 64) attn_prefill_kernel<64, 2><<<grid, 256, 0, s>>>(a);
   else if (head_dim == 128) attn_prefill_kernel<128, 2><<<grid, 256, 0, s>>>(a);
   else attn_prefill_kernel<256, 1><<<grid, 256, 0, s>>>(a);
+  HOLON_LAUNCH_OK();
+  return 0;
+}
+
+// Prompt portions of windowed attention with sigmoid weights (head sizes 64 and 128, keys and values of one width,
+// groups of up to 32 heads): the wide prompt kernel with the softmax taken out.
+extern "C" int holon_sigmoid_attention_prefill_bf16(const void* q, void* out, const void* pages, const int32_t* table,
+                                                    int table_stride, const int32_t* slots, const int32_t* lens,
+                                                    const int32_t* query_start, const int32_t* row_ids, int n_rows,
+                                                    int max_query, int max_len, int heads, int kv_heads, int head_dim,
+                                                    int page_size, float scale, int window, const float* head_bias,
+                                                    const void* gate, void* stream) {
+  HOLON_CHECK((head_dim == 64 || head_dim == 128) && mfma_serves(head_dim, page_size),
+              "sigmoid attention (matrix cores): head_dim %d / page %d not served", head_dim, page_size);
+  HOLON_CHECK(heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && heads / kv_heads <= 32 && window >= 0 &&
+              table_stride > 0 && max_len <= 4096 * page_size, "sigmoid attention: bad sizes");
+  if (n_rows <= 0 || max_query <= 0) return 0;
+  AttnArgs a{};
+  a.q = (const bf16_t*)q; a.out = (bf16_t*)out; a.pages = (const bf16_t*)pages; a.table = table;
+  a.table_stride = table_stride; a.slots = slots; a.lens = lens; a.qstart = query_start; a.row_ids = row_ids;
+  a.heads = heads; a.kv_heads = kv_heads; a.page_size = page_size; a.window = window;
+  a.scale = scale; a.head_bias = head_bias; a.gate = (const bf16_t*)gate;
+  const TileMap32 tm32 = tile_map32(heads / kv_heads);
+  const int ranges32 = ((max_query + tm32.pos_per_tile - 1) / tm32.pos_per_tile + 3) / 4;
+  a.unpaired = (int64_t)((ranges32 + 1) / 2) * kv_heads * n_rows < UNPAIR_BELOW ? 1 : 0;
+  dim3 grid(kv_heads, (ranges32 + 1) / 2, a.unpaired ? 2 * n_rows : n_rows);
+  HOLON_CHECK(grid.y <= 65535 && grid.z <= 65535, "sigmoid attention: %d rows of %d tokens exceed one launch", n_rows,
+              max_query);
+  if (head_dim == 64) attn_prefill_wide_kernel<64, true><<<grid, 256, 0, (hipStream_t)stream>>>(a);
+  else attn_prefill_wide_kernel<128, true><<<grid, 256, 0, (hipStream_t)stream>>>(a);
   HOLON_LAUNCH_OK();
   return 0;
 }

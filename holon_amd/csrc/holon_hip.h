@@ -213,15 +213,22 @@ int holon_shift_mix(const void* x, const void* mu, void* state, void* y, const i
 int holon_decay_lora(const float* a, const void* w2, const float* w0, float* y, int tokens, int channels, int rank,
                      int dtype, void* stream);
 
-// -- windowed sigmoid attention (sigmoid_attention.hip); a page is keys [Hkv, P, D] then values [Hkv, P, V] ---------------
+// -- windowed sigmoid attention (sigmoid_attention.hip); a page is keys [Hkv, P, D] then values [Hkv, V, P] ---------------
 int holon_head_prepare(const void* qkv, void* q_out, int tokens, int heads, int kv_heads, int dim, int vdim,
                        const void* q_weight, const void* k_weight, float eps, const float* table, int rot, int table_rows,
                        const int32_t* positions, void* pages, const int32_t* write_page, const int32_t* write_off,
                        int page_size, int num_pages, int dtype, void* stream);
 int holon_sigmoid_attention(const void* q, void* out, const void* pages, const int32_t* table, int table_stride,
-                            const int32_t* slots, const int32_t* token_row, const int32_t* positions, int tokens,
-                            int heads, int kv_heads, int dim, int vdim, int page_size, int num_pages, const float* bias,
-                            float scale, int window, const void* gate, int dtype, void* stream);
+                            const int32_t* slots, const int32_t* token_row, const int32_t* positions,
+                            const int32_t* query_start, const int32_t* row_ids, int tokens, int heads, int kv_heads,
+                            int dim, int vdim, int page_size, int num_pages, const float* bias, float scale, int window,
+                            const void* gate, int dtype, void* stream);
+// The prompt portions (rows listed in row_ids) on the matrix cores: bfloat16, keys and values of one width 64 or 128.
+int holon_sigmoid_attention_prefill_bf16(const void* q, void* out, const void* pages, const int32_t* table,
+                                         int table_stride, const int32_t* slots, const int32_t* lens,
+                                         const int32_t* query_start, const int32_t* row_ids, int n_rows, int max_query,
+                                         int max_len, int heads, int kv_heads, int head_dim, int page_size, float scale,
+                                         int window, const float* head_bias, const void* gate, void* stream);
 
 #ifdef __cplusplus
 }

@@ -3,10 +3,11 @@
 // (query_start[b] .. query_start[b + 1]), each continuing the state in its request's slot; a row that starts at
 // position 0 starts from zeros whatever the slot holds.
 //
-// The two scans keep, per (row, head), one thread per value column j of the head's matrix S [D, V]: the columns never
-// meet, so a thread carries its D values in registers through the row's tokens; a block is one wave of 64 columns,
-// which shares each token's key and query through LDS. The key size is padded to the next instantiated one with zeros (a zero key writes nothing).
-// Every sum runs over the key index in ascending order.
+// The two scans keep a head's matrix S [D, V] in registers through a row's tokens. Its columns never meet, so a wave
+// owns 16 of them, four lanes a column with a quarter of the key rows each; what a token needs of a whole column (a dot
+// product with the key, the read-out) is summed over a lane's rows in ascending order and then over the four lanes in a
+// fixed order. Each token's key and query reach the lanes through LDS. The key size is padded to the next instantiated
+// one with zeros (a zero key writes nothing).
 #include "common.h"
 #include "holon_hip.h"
 
@@ -97,95 +98,153 @@ __global__ void __launch_bounds__(256) delta_prepare_kernel(const T* __restrict_
   }
 }
 
-// Per (row, head): S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q. Thread j owns column j of S.
+// Sum over the four adjacent lanes that share a column (a fixed order: lane ^ 1, then lane ^ 2).
+__device__ __forceinline__ float quad_sum(float v) {
+  v += __shfl_xor(v, 1, WAVE);
+  v += __shfl_xor(v, 2, WAVE);
+  return v;
+}
+
+constexpr int SCAN_COLS = 16;      // value columns a wave owns; four lanes a column, each a quarter of the key rows
+
+// Per (row, head): S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q. Lane 4 c + p owns rows
+// p KD/4 .. (p + 1) KD/4 - 1 of column c of S. The next token's operands are asked for before this token's arithmetic.
 template <int KD, typename T>
-__global__ void __launch_bounds__(WAVE) delta_scan_kernel(const float* __restrict__ qn, const float* __restrict__ kn, const T* __restrict__ qkv,
-                                  int qkv_stride, int v_offset, const float* __restrict__ beta,
-                                  const float* __restrict__ g, float* __restrict__ state, float* __restrict__ out,
-                                  const int32_t* __restrict__ slots, const int32_t* __restrict__ starts,
-                                  const int32_t* __restrict__ query_start, int heads, int kv_heads, int dim, int vdim) {
+__global__ void __launch_bounds__(WAVE) delta_scan_kernel(const float* __restrict__ qn, const float* __restrict__ kn,
+                                                          const T* __restrict__ qkv, int qkv_stride, int v_offset,
+                                                          const float* __restrict__ beta, const float* __restrict__ g,
+                                                          float* __restrict__ state, float* __restrict__ out,
+                                                          const int32_t* __restrict__ slots,
+                                                          const int32_t* __restrict__ starts,
+                                                          const int32_t* __restrict__ query_start, int heads,
+                                                          int kv_heads, int dim, int vdim) {
+  constexpr int KQ = KD / 4, PER = (KD + WAVE - 1) / WAVE;
   __shared__ float ks[KD], qs[KD];
-  const int b = blockIdx.x, h = blockIdx.y, j = blockIdx.z * WAVE + threadIdx.x;
+  const int b = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int part = lane % 4, j = blockIdx.z * SCAN_COLS + lane / 4;
   const int hk = h / (heads / kv_heads);
   const bool active = j < vdim;
   const int lo = query_start[b], hi = query_start[b + 1];
   float* held = state + ((int64_t)slots[b] * heads + h) * dim * vdim;
   const bool carried = starts[b] > 0;
-  float S[KD];
+  float S[KQ];
 #pragma unroll
-  for (int i = 0; i < KD; ++i) S[i] = (carried && active && i < dim) ? held[(int64_t)i * vdim + j] : 0.f;
+  for (int i = 0; i < KQ; ++i) {
+    const int row = part * KQ + i;
+    S[i] = (carried && active && row < dim) ? held[(int64_t)row * vdim + j] : 0.f;
+  }
+  float nk[PER], nq[PER], ng = 0.f, nb = 0.f, nv = 0.f;
+  auto ask = [&](int t) {
+#pragma unroll
+    for (int e = 0; e < PER; ++e) {
+      const int i = lane + e * WAVE;
+      nk[e] = i < dim ? kn[((int64_t)t * kv_heads + hk) * dim + i] : 0.f;
+      nq[e] = i < dim ? qn[((int64_t)t * kv_heads + hk) * dim + i] : 0.f;
+    }
+    ng = g[(int64_t)t * heads + h];
+    nb = beta[(int64_t)t * heads + h];
+    nv = active ? Elem<T>::load(qkv[(int64_t)t * qkv_stride + v_offset + h * vdim + j]) : 0.f;
+  };
+  if (lo < hi) ask(lo);
   for (int t = lo; t < hi; ++t) {
     __syncthreads();
-    for (int i = threadIdx.x; i < KD; i += blockDim.x) {
-      ks[i] = i < dim ? kn[((int64_t)t * kv_heads + hk) * dim + i] : 0.f;
-      qs[i] = i < dim ? qn[((int64_t)t * kv_heads + hk) * dim + i] : 0.f;
+#pragma unroll
+    for (int e = 0; e < PER; ++e) {
+      const int i = lane + e * WAVE;
+      if (i < KD) { ks[i] = nk[e]; qs[i] = nq[e]; }
     }
+    const float gt = ng, bt = nb, vt = nv;
     __syncthreads();
-    const float gt = g[(int64_t)t * heads + h], bt = beta[(int64_t)t * heads + h];
-    const float vt = active ? Elem<T>::load(qkv[(int64_t)t * qkv_stride + v_offset + h * vdim + j]) : 0.f;
+    if (t + 1 < hi) ask(t + 1);
     float dot = 0.f;
 #pragma unroll
-    for (int i = 0; i < KD; ++i) {
+    for (int i = 0; i < KQ; ++i) {
       S[i] *= gt;
-      dot += S[i] * ks[i];
+      dot += S[i] * ks[part * KQ + i];
     }
-    const float u = bt * (vt - dot);
+    const float u = bt * (vt - quad_sum(dot));
     float o = 0.f;
 #pragma unroll
-    for (int i = 0; i < KD; ++i) {
-      S[i] += ks[i] * u;
-      o += S[i] * qs[i];
+    for (int i = 0; i < KQ; ++i) {
+      S[i] += ks[part * KQ + i] * u;
+      o += S[i] * qs[part * KQ + i];
     }
-    if (active) out[((int64_t)t * heads + h) * vdim + j] = o;
+    o = quad_sum(o);
+    if (active && part == 0) out[((int64_t)t * heads + h) * vdim + j] = o;
   }
   if (active) {
 #pragma unroll
-    for (int i = 0; i < KD; ++i)
-      if (i < dim) held[(int64_t)i * vdim + j] = S[i];
+    for (int i = 0; i < KQ; ++i) {
+      const int row = part * KQ + i;
+      if (row < dim) held[(int64_t)row * vdim + j] = S[i];
+    }
   }
 }
 
-// Per (row, head): o = (S + diag(u) k v^T)^T r; S <- diag(w) S + k v^T. Thread j owns column j of S [D, D].
+// Per (row, head): o = (S + diag(u) k v^T)^T r; S <- diag(w) S + k v^T. The same split of S [D, D] over lanes.
 template <int KD, typename T>
-__global__ void __launch_bounds__(WAVE) memory_scan_kernel(const T* __restrict__ r, const T* __restrict__ k, const T* __restrict__ v,
-                                   const float* __restrict__ w, const float* __restrict__ u, float* __restrict__ state,
-                                   float* __restrict__ out, const int32_t* __restrict__ slots,
-                                   const int32_t* __restrict__ starts, const int32_t* __restrict__ query_start,
-                                   int heads, int dim) {
+__global__ void __launch_bounds__(WAVE) memory_scan_kernel(const T* __restrict__ r, const T* __restrict__ k,
+                                                           const T* __restrict__ v, const float* __restrict__ w,
+                                                           const float* __restrict__ u, float* __restrict__ state,
+                                                           float* __restrict__ out, const int32_t* __restrict__ slots,
+                                                           const int32_t* __restrict__ starts,
+                                                           const int32_t* __restrict__ query_start, int heads, int dim) {
+  constexpr int KQ = KD / 4, PER = (KD + WAVE - 1) / WAVE;
   __shared__ float rs[KD], ks[KD], ws[KD], us[KD];
-  const int b = blockIdx.x, h = blockIdx.y, j = blockIdx.z * WAVE + threadIdx.x;
+  const int b = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int part = lane % 4, j = blockIdx.z * SCAN_COLS + lane / 4;
   const bool active = j < dim;
   const int lo = query_start[b], hi = query_start[b + 1];
   float* held = state + ((int64_t)slots[b] * heads + h) * dim * dim;
   const bool carried = starts[b] > 0;
-  float S[KD];
+  float S[KQ];
 #pragma unroll
-  for (int i = 0; i < KD; ++i) S[i] = (carried && active && i < dim) ? held[(int64_t)i * dim + j] : 0.f;
-  for (int i = threadIdx.x; i < KD; i += blockDim.x) us[i] = i < dim ? u[h * dim + i] : 0.f;
+  for (int i = 0; i < KQ; ++i) {
+    const int row = part * KQ + i;
+    S[i] = (carried && active && row < dim) ? held[(int64_t)row * dim + j] : 0.f;
+  }
+  for (int i = lane; i < KD; i += WAVE) us[i] = i < dim ? u[h * dim + i] : 0.f;
   const int64_t width = (int64_t)heads * dim;
+  float nr[PER], nk[PER], nw[PER], nv = 0.f;
+  auto ask = [&](int t) {
+#pragma unroll
+    for (int e = 0; e < PER; ++e) {
+      const int i = lane + e * WAVE;
+      const int64_t at = (int64_t)t * width + h * dim + i;
+      nr[e] = i < dim ? Elem<T>::load(r[at]) : 0.f;
+      nk[e] = i < dim ? Elem<T>::load(k[at]) : 0.f;
+      nw[e] = i < dim ? w[at] : 0.f;
+    }
+    nv = active ? Elem<T>::load(v[(int64_t)t * width + h * dim + j]) : 0.f;
+  };
+  if (lo < hi) ask(lo);
   for (int t = lo; t < hi; ++t) {
     __syncthreads();
-    for (int i = threadIdx.x; i < KD; i += blockDim.x) {
-      const int64_t at = (int64_t)t * width + h * dim + i;
-      rs[i] = i < dim ? Elem<T>::load(r[at]) : 0.f;
-      ks[i] = i < dim ? Elem<T>::load(k[at]) : 0.f;
-      ws[i] = i < dim ? w[at] : 0.f;
+#pragma unroll
+    for (int e = 0; e < PER; ++e) {
+      const int i = lane + e * WAVE;
+      if (i < KD) { rs[i] = nr[e]; ks[i] = nk[e]; ws[i] = nw[e]; }
     }
+    const float vt = nv;
     __syncthreads();
-    const float vt = active ? Elem<T>::load(v[(int64_t)t * width + h * dim + j]) : 0.f;
+    if (t + 1 < hi) ask(t + 1);
     float o = 0.f;
 #pragma unroll
-    for (int i = 0; i < KD; ++i) {
-      const float kv = ks[i] * vt;
-      o += rs[i] * (S[i] + us[i] * kv);
-      S[i] = ws[i] * S[i] + kv;
+    for (int i = 0; i < KQ; ++i) {
+      const int row = part * KQ + i;
+      const float kv = ks[row] * vt;
+      o += rs[row] * (S[i] + us[row] * kv);
+      S[i] = ws[row] * S[i] + kv;
     }
-    if (active) out[(int64_t)t * width + h * dim + j] = o;
+    o = quad_sum(o);
+    if (active && part == 0) out[(int64_t)t * width + h * dim + j] = o;
   }
   if (active) {
 #pragma unroll
-    for (int i = 0; i < KD; ++i)
-      if (i < dim) held[(int64_t)i * dim + j] = S[i];
+    for (int i = 0; i < KQ; ++i) {
+      const int row = part * KQ + i;
+      if (row < dim) held[(int64_t)row * dim + j] = S[i];
+    }
   }
 }
 
@@ -325,7 +384,7 @@ extern "C" int holon_delta_scan(const float* qn, const float* kn, const void* qk
   HOLON_CHECK(rows <= 0x7fffffff / 2 && heads <= 65535 && state_slots > 0 && v_offset >= 0 &&
               v_offset + heads * vdim <= qkv_stride, "delta_scan: launch or row layout out of range");
   if (rows == 0) return 0;
-  const dim3 grid(rows, heads, (vdim + WAVE - 1) / WAVE);     // a wave for every 64 value columns
+  const dim3 grid(rows, heads, (vdim + SCAN_COLS - 1) / SCAN_COLS);     // a wave for every 16 value columns
   hipStream_t s = (hipStream_t)stream;
   BY_DTYPE(dtype, BY_KEY_SIZE(dim, (launch_delta<T, KD>(grid, s, qn, kn, qkv, qkv_stride, v_offset, beta, g,
                                                          state, out, slots, starts, query_start, heads, kv_heads, dim,
@@ -349,7 +408,7 @@ extern "C" int holon_memory_scan(const void* r, const void* k, const void* v, co
   HOLON_CHECK(rows >= 0 && heads > 0 && heads <= 65535 && dim > 0 && dim <= 256 && state_slots > 0,
               "memory_scan: %d heads of %d (at most 256)", heads, dim);
   if (rows == 0) return 0;
-  const dim3 grid(rows, heads, (dim + WAVE - 1) / WAVE);
+  const dim3 grid(rows, heads, (dim + SCAN_COLS - 1) / SCAN_COLS);
   hipStream_t s = (hipStream_t)stream;
   BY_DTYPE(dtype, BY_KEY_SIZE(dim, (launch_memory<T, KD>(grid, s, r, k, v, w, u, state, out, slots, starts,
                                                           query_start, heads, dim))));

@@ -1,6 +1,8 @@
 // Windowed attention with sigmoid weights over a paged cache whose keys and values may differ in width.
 //
-// One page of one site holds P tokens: keys [Hkv, P, D] followed by values [Hkv, P, V], token-major. `head_prepare`
+// One page of one site holds P tokens: keys [Hkv, P, D] (a token's key is a row) followed by values [Hkv, V, P]
+// (transposed inside the page: a matrix-core operand of the value product is then one contiguous load; with V = D this
+// is the layout of the framework's softmax attention). `head_prepare`
 // norms and rotates the heads of a merged q/k/v projection and stores keys and values; `sigmoid_attention` sums
 // sigmoid(q . k * scale + bias) * v over the keys a query sees. Nothing is normalised over keys, so there is no running
 // maximum and no rescaling: a query's result is a plain sum, taken over its keys from the oldest visible one on, in
@@ -36,8 +38,8 @@ __global__ void __launch_bounds__(256) head_prepare_kernel(const T* __restrict__
     const int hv = hs - heads - kv_heads;
     if (!page_ok) return;
     const T* src = row + (int64_t)(heads + kv_heads) * dim + (int64_t)hv * vdim;
-    T* dst = pages + page * page_len + (int64_t)kv_heads * page_size * dim + ((int64_t)hv * page_size + off) * vdim;
-    for (int d = lane; d < vdim; d += WAVE) dst[d] = src[d];
+    T* dst = pages + page * page_len + (int64_t)kv_heads * page_size * dim + (int64_t)hv * vdim * page_size + off;
+    for (int d = lane; d < vdim; d += WAVE) dst[(int64_t)d * page_size] = src[d];
     return;
   }
   const bool is_q = hs < heads;
@@ -72,7 +74,8 @@ __global__ void __launch_bounds__(256) head_prepare_kernel(const T* __restrict__
     dst[d] = Elem<T>::store(Elem<T>::load(src[d]) * r * (w ? Elem<T>::load(w[d]) : 1.f));
 }
 
-// One wave per (token, head), four heads of a token per block. A lane takes one key of a tile of 64: its score over D
+// The general kernel (any dtype and sizes; the decode rows of every step): one wave per (token, head), four heads of
+// a token per block. A lane takes one key of a tile of 64: its score over D
 // (the query comes from LDS), its weight; then the lanes turn to the value columns and add the tile's weighted values.
 template <typename T, bool VEC>
 __global__ void __launch_bounds__(256) sigmoid_attention_kernel(const T* __restrict__ q, T* __restrict__ out,
@@ -80,7 +83,9 @@ __global__ void __launch_bounds__(256) sigmoid_attention_kernel(const T* __restr
                                                                 const int32_t* __restrict__ table, int table_stride,
                                                                 const int32_t* __restrict__ slots,
                                                                 const int32_t* __restrict__ token_row,
-                                                                const int32_t* __restrict__ positions, int heads,
+                                                                const int32_t* __restrict__ positions,
+                                                                const int32_t* __restrict__ query_start,
+                                                                const int32_t* __restrict__ row_ids, int heads,
                                                                 int kv_heads, int dim, int vdim, int page_size,
                                                                 const float* __restrict__ bias, float scale, int window,
                                                                 const T* __restrict__ gate) {
@@ -88,7 +93,7 @@ __global__ void __launch_bounds__(256) sigmoid_attention_kernel(const T* __restr
   __shared__ float p_s[4][WAVE];
   __shared__ int64_t v_s[4][WAVE];
   const int w = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
-  const int t = blockIdx.x;
+  const int t = row_ids ? query_start[row_ids[blockIdx.x]] : blockIdx.x;   // the one token of a listed row, or every token
   const bool live = blockIdx.y * 4 + w < heads;
   const int h = live ? blockIdx.y * 4 + w : 0;       // a spare wave walks head 0 and stores nothing: all reach the barriers
   const int pos = positions[t];
@@ -114,7 +119,7 @@ __global__ void __launch_bounds__(256) sigmoid_attention_kernel(const T* __restr
       const int page = trow[key / page_size];
       const int off = key - (key / page_size) * page_size;
       const T* kp = pages + page * page_len + ((int64_t)hk * page_size + off) * dim;
-      voff = page * page_len + val_base + ((int64_t)hk * page_size + off) * vdim;
+      voff = page * page_len + val_base + (int64_t)hk * vdim * page_size + off;
       float dot = 0.f;
       if (VEC) {
         for (int d = 0; d < dim; d += V) {
@@ -137,7 +142,7 @@ __global__ void __launch_bounds__(256) sigmoid_attention_kernel(const T* __restr
       const int d = lane + i * WAVE;
       if (d < vdim) {
         float a = acc[i];
-        for (int j = 0; j < count; ++j) a += p_s[w][j] * Elem<T>::load(pages[v_s[w][j] + d]);
+        for (int j = 0; j < count; ++j) a += p_s[w][j] * Elem<T>::load(pages[v_s[w][j] + (int64_t)d * page_size]);
         acc[i] = a;
       }
     }
@@ -187,23 +192,26 @@ extern "C" int holon_head_prepare(const void* qkv, void* q_out, int tokens, int 
 
 extern "C" int holon_sigmoid_attention(const void* q, void* out, const void* pages, const int32_t* table,
                                        int table_stride, const int32_t* slots, const int32_t* token_row,
-                                       const int32_t* positions, int tokens, int heads, int kv_heads, int dim, int vdim,
-                                       int page_size, int num_pages, const float* bias, float scale, int window,
-                                       const void* gate, int dtype, void* stream) {
+                                       const int32_t* positions, const int32_t* query_start, const int32_t* row_ids,
+                                       int tokens, int heads, int kv_heads, int dim, int vdim, int page_size,
+                                       int num_pages, const float* bias, float scale, int window, const void* gate,
+                                       int dtype, void* stream) {
   HOLON_CHECK(tokens >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "sigmoid_attention: %d/%d heads", heads,
               kv_heads);
   HOLON_CHECK(dim > 0 && dim <= SIG_MAX_D && vdim > 0 && vdim <= SIG_MAX_D,
               "sigmoid_attention: head sizes %d/%d (at most %d)", dim, vdim, SIG_MAX_D);
   HOLON_CHECK(page_size > 0 && num_pages > 0 && window >= 0 && table_stride > 0, "sigmoid_attention: bad page geometry");
-  if (tokens == 0) return 0;
+  HOLON_CHECK(row_ids == nullptr || query_start != nullptr, "sigmoid_attention: listed rows need query_start");
+  if (tokens == 0) return 0;        // (with row_ids: `tokens` is the number of listed rows)
   const dim3 grid(tokens, (heads + 3) / 4);
   hipStream_t s = (hipStream_t)stream;
   const int vec = dtype == HOLON_F32 ? 4 : 8;
-  const bool aligned = dim % vec == 0 && vdim % vec == 0 && (uintptr_t)pages % 16 == 0;
+  const bool aligned = dim % vec == 0 && ((int64_t)vdim * page_size) % vec == 0 && (uintptr_t)pages % 16 == 0;
 #define SIG_LAUNCH(T, VEC)                                                                                            \
   sigmoid_attention_kernel<T, VEC><<<grid, 256, 0, s>>>((const T*)q, (T*)out, (const T*)pages, table, table_stride,  \
-                                                        slots, token_row, positions, heads, kv_heads, dim, vdim,     \
-                                                        page_size, bias, scale, window, (const T*)gate)
+                                                        slots, token_row, positions, query_start, row_ids, heads,     \
+                                                        kv_heads, dim, vdim, page_size, bias, scale, window,         \
+                                                        (const T*)gate)
   if (dtype == HOLON_F32) { if (aligned) SIG_LAUNCH(float, true); else SIG_LAUNCH(float, false); }
   else { if (aligned) SIG_LAUNCH(bf16_t, true); else SIG_LAUNCH(bf16_t, false); }
 #undef SIG_LAUNCH

@@ -125,6 +125,7 @@ class HipKernels:
 
     # -- operations that parts bring with them ----------------------------------------------------------------------
     _part_libs: dict[str, ctypes.CDLL] = {}       # libraries built from parts' own sources, by source path
+    _bound: dict[str, tuple] = {}                 # operation name -> (its registration, the bound call)
 
     def __getattr__(self, name: str):
         """An operation registered with `holon_amd.kernels.registry.register_kernel`: its HIP form when it has one
@@ -135,6 +136,9 @@ class HipKernels:
             raise AttributeError(f"{type(self).__name__} has no operation {name!r}")
         if op.symbol is None:
             return op.plain
+        bound = self._bound.get(name)
+        if bound is not None and bound[0] is op:      # bound before (the same registration)
+            return bound[1]
         lib = self.lib
         if op.source is not None:
             key = str(op.source)
@@ -145,15 +149,24 @@ class HipKernels:
                     lib = self._part_libs[key] = ctypes.CDLL(str(path))
                 except OSError as e:
                     raise KernelError(f"cannot load {path}: {e}") from e
-        fn = getattr(lib, op.symbol)
-        fn.argtypes, fn.restype = [*op.argtypes, _P], _I
 
-        def launch(*args) -> None:
-            rc = fn(*args, self._stream())
-            if rc != 0:
-                detail = self.lib.holon_last_error().decode() if op.source is None else f"returned {rc}"
-                raise KernelError(f"{op.symbol}: {detail}")
-        return lambda *args, **kwargs: op.call(launch, *args, **kwargs)
+        def bind(symbol, argtypes):
+            fn = getattr(lib, symbol)
+            fn.argtypes, fn.restype = [*argtypes, _P], _I
+
+            def launch(*args) -> None:
+                rc = fn(*args, self._stream())
+                if rc != 0:
+                    detail = self.lib.holon_last_error().decode() if op.source is None else f"returned {rc}"
+                    raise KernelError(f"{symbol}: {detail}")
+            return launch
+        if isinstance(op.symbol, tuple):          # several entry points behind one operation
+            launch = tuple(bind(sym, types) for sym, types in zip(op.symbol, op.argtypes, strict=True))
+        else:
+            launch = bind(op.symbol, op.argtypes)
+        call = lambda *args, **kwargs: op.call(launch, *args, **kwargs)      # noqa: E731
+        self._bound[name] = (op, call)
+        return call
 
     # -- plumbing -------------------------------------------------------------------------------------------------
     def _call(self, fn, *args) -> None:

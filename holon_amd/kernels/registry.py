@@ -14,7 +14,9 @@ symbol is built from when it is not part of this package's own library. Every ke
         call=lambda launch, x, state, ...: launch(x.data_ptr(), state.data_ptr(), ...)))
 
 `call` gets `launch(*c_args)`, which appends the current HIP stream as the last argument, calls the symbol and raises
-`KernelError` when it returns non-zero; the function returns what the operation returns. The source is compiled for
+`KernelError` when it returns non-zero; the function returns what the operation returns. An operation that runs
+several entry points names them all: `symbol` a tuple of names, `argtypes` a tuple of their lists, and `call` gets a
+tuple of launchers in the same order. The source is compiled for
 gfx950 with this package's flags into `lib<stem>.so` beside it (or, where that folder cannot be written, into the
 per-user build folder) the first time the operation is called and no such library is there;
 `holon_amd.kernels.build.build_source` builds it ahead of time.
@@ -31,8 +33,9 @@ from typing import Any
 class KernelOp:
     name: str
     plain: Callable[..., Any]
-    symbol: str | None = None
-    argtypes: Sequence[Any] = ()                  # without the trailing stream (a void pointer), which `launch` adds
+    symbol: "str | tuple[str, ...] | None" = None
+    argtypes: Sequence[Any] = ()                  # without the trailing stream (a void pointer), which `launch` adds;
+                                                  # with several symbols: one list for each
     call: Callable[..., Any] | None = None
     source: str | pathlib.Path | None = None      # None: the symbol is in libholon_hip.so
 

@@ -2,9 +2,11 @@
 sigmoid(q_i . k_j * scale + bias[head]) * v_j to query i, and nothing is normalised over keys. Query i sees keys
 i - window + 1 .. i (window 0: all before it). Scores and weights are float32.
 
-Keys and values live in the paged cache with a layout of this mixer's own, since keys and values may differ in
-width: one page of one site is `[Hkv, P, D]` keys followed by `[Hkv, P, V]` values, token-major.
-HIP forms: `csrc/sigmoid_attention.hip`."""
+Keys and values may differ in width. One page of one site is `[Hkv, P, D]` keys (a token's key is a row) followed by
+`[Hkv, V, P]` values (transposed inside the page); with V = D this is the layout of the softmax attention's pages.
+HIP forms: `csrc/sigmoid_attention.hip` (any dtype and sizes, and the decode rows of every step) and, for prompt
+portions in bfloat16 with keys and values of one width 64 or 128, the matrix-core prompt kernel of
+`csrc/attention_mfma.hip` with sigmoid weights in place of its softmax."""
 from __future__ import annotations
 
 import ctypes
@@ -30,7 +32,8 @@ def head_prepare_plain(qkv, heads, kv_heads, dim, vdim, q_weight, k_weight, eps,
     """qkv [T, (H + G) D + G V] (queries, keys, values side by side). Per head of q and k: x * rsqrt(mean(x^2) + eps)
     * weight (when weights are given), then the rotation by `table` [positions, rot] (cos of rot/2 angles, then
     their sines; pairs (i, i + rot/2); dimensions from rot on pass), all in float32 with one rounding. Keys and
-    values go into `pages` [pages, G P (D + V)] at (write_page[t], write_off[t]); returns q [T, H, D]."""
+    values go into `pages` [pages, G P (D + V)] (keys [G, P, D], then values [G, V, P]) at (write_page[t],
+    write_off[t]); returns q [T, H, D]."""
     t = qkv.shape[0]
     q = qkv[:, : heads * dim].float().view(t, heads, dim)
     k = qkv[:, heads * dim: (heads + kv_heads) * dim].float().view(t, kv_heads, dim)
@@ -48,9 +51,9 @@ def head_prepare_plain(qkv, heads, kv_heads, dim, vdim, q_weight, k_weight, eps,
             return torch.cat((a * cos - b * sin, b * cos + a * sin, x[..., rot:]), dim=-1)
         q, k = turn(q), turn(k)
     keys = pages[:, : kv_heads * page_size * dim].view(-1, kv_heads, page_size, dim)
-    vals = pages[:, kv_heads * page_size * dim:].view(-1, kv_heads, page_size, vdim)
+    vals = pages[:, kv_heads * page_size * dim:].view(-1, kv_heads, vdim, page_size)
     keys[write_page.long(), :, write_off.long()] = k.to(pages.dtype)
-    vals[write_page.long(), :, write_off.long()] = v.to(pages.dtype)
+    vals[write_page.long(), :, :, write_off.long()] = v.to(pages.dtype)
     return q.to(qkv.dtype)
 
 
@@ -75,17 +78,18 @@ def _head_prepare_hip(launch, qkv, heads, kv_heads, dim, vdim, q_weight, k_weigh
     return q
 
 
-def sigmoid_attention_plain(q, pages, table, slots, token_row, positions, kv_heads, vdim, page_size, bias, scale,
+def sigmoid_attention_plain(q, pages, table, rows, token_row, positions, kv_heads, vdim, page_size, bias, scale,
                             window, gate):
-    """q [T, H, D]; `pages` as `head_prepare` writes them; `table` [S, max_pages] int32; token t belongs to row
-    token_row[t] (slot slots[row]) and stands at positions[t]. bias [H] float32 or None. `gate` [T, H V] or None:
-    the result is multiplied by sigmoid(gate). -> [T, H V] in q's dtype; the sum over keys runs oldest first."""
+    """q [T, H, D]; `pages` as `head_prepare` writes them; `table` [S, max_pages] int32; `rows`: the step's rows
+    (`AttnRows`); token t belongs to row token_row[t] (slot rows.slots[row]) and stands at positions[t]. bias [H]
+    float32 or None. `gate` [T, H V] or None: the result is multiplied by sigmoid(gate). -> [T, H V] in q's dtype;
+    the sum over keys runs oldest first."""
     t, heads, dim = q.shape
     keys = pages[:, : kv_heads * page_size * dim].view(-1, kv_heads, page_size, dim)
-    vals = pages[:, kv_heads * page_size * dim:].view(-1, kv_heads, page_size, vdim)
+    vals = pages[:, kv_heads * page_size * dim:].view(-1, kv_heads, vdim, page_size).transpose(2, 3)
     out = torch.zeros((t, heads, vdim), dtype=torch.float32, device=q.device)
-    rows, pos = token_row.tolist(), positions.tolist()
-    slot_of = slots.tolist()
+    pos = positions.tolist()
+    slot_of, rows = rows.slots.tolist(), token_row.tolist()
     group = heads // kv_heads
     for i in range(t):
         first = max(0, pos[i] - window + 1) if window > 0 else 0
@@ -106,7 +110,7 @@ def sigmoid_attention_plain(q, pages, table, slots, token_row, positions, kv_hea
     return out.to(q.dtype)
 
 
-def _sigmoid_attention_hip(launch, q, pages, table, slots, token_row, positions, kv_heads, vdim, page_size, bias,
+def _sigmoid_attention_hip(launch, q, pages, table, rows, token_row, positions, kv_heads, vdim, page_size, bias,
                            scale, window, gate):
     t, heads, dim = q.shape
     ok = q.is_cuda and q.is_contiguous() and q.dtype in _DT and pages.dtype == q.dtype and pages.is_contiguous() \
@@ -118,17 +122,31 @@ def _sigmoid_attention_hip(launch, q, pages, table, slots, token_row, positions,
         raise ValueError(f"sigmoid_attention: q {tuple(q.shape)} {q.dtype}, pages {tuple(pages.shape)} do not fit "
                          f"{kv_heads} kv heads, values of {vdim}, page {page_size}")
     out = torch.empty((t, heads * vdim), dtype=q.dtype, device=q.device)
-    launch(q.data_ptr(), out.data_ptr(), pages.data_ptr(), table.data_ptr(), table.shape[1], slots.data_ptr(),
-           token_row.data_ptr(), positions.data_ptr(), t, heads, kv_heads, dim, vdim, page_size, pages.shape[0],
-           _ptr(bias), float(scale), int(window), _ptr(gate), _DT[q.dtype])
+    general, wide = launch
+    common = (q.data_ptr(), out.data_ptr(), pages.data_ptr(), table.data_ptr(), table.shape[1], rows.slots.data_ptr())
+    tail = (heads, kv_heads, dim, vdim, page_size, pages.shape[0], _ptr(bias), float(scale), int(window), _ptr(gate),
+            _DT[q.dtype])
+    on_cores = q.dtype == torch.bfloat16 and dim == vdim and dim in (64, 128) and page_size % 16 == 0 \
+        and heads // kv_heads <= 32 and rows.n_chunk > 0 and rows.max_chunk_len <= 4096 * page_size
+    if on_cores:      # prompt portions on the matrix cores, the step's decode rows (if any) in the general kernel
+        wide(*common, rows.lens.data_ptr(), rows.query_start.data_ptr(), rows.chunk_rows.data_ptr(), rows.n_chunk,
+             rows.max_chunk_query, rows.max_chunk_len, heads, kv_heads, dim, page_size, float(scale), int(window),
+             _ptr(bias), _ptr(gate))
+        if rows.n_decode:
+            general(*common, token_row.data_ptr(), positions.data_ptr(), rows.query_start.data_ptr(),
+                    rows.decode_rows.data_ptr(), rows.n_decode, *tail)
+    else:
+        general(*common, token_row.data_ptr(), positions.data_ptr(), None, None, t, *tail)
     return out
 
 
 register_kernel(KernelOp("head_prepare", head_prepare_plain, "holon_head_prepare",
                          [_P, _P, _I, _I, _I, _I, _I, _P, _P, _F, _P, _I, _I, _P, _P, _P, _P, _I, _I, _I],
                          _head_prepare_hip))
-register_kernel(KernelOp("sigmoid_attention", sigmoid_attention_plain, "holon_sigmoid_attention",
-                         [_P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P, _F, _I, _P, _I],
+register_kernel(KernelOp("sigmoid_attention", sigmoid_attention_plain,
+                         ("holon_sigmoid_attention", "holon_sigmoid_attention_prefill_bf16"),
+                         ([_P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P, _F, _I, _P, _I],
+                          [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P, _P]),
                          _sigmoid_attention_hip))
 
 
@@ -191,7 +209,7 @@ class SigmoidWindowAttention(Part):
                            self.eps or 0.0, table, step.positions, held.pages, view.write_page, view.write_off,
                            view.page_size)
         gate = self.g(x) if self.g is not None else None
-        out = k.sigmoid_attention(q, held.pages, view.table, step.slots, step.token_row, step.positions,
+        out = k.sigmoid_attention(q, held.pages, view.table, step.rows, step.token_row, step.positions,
                                   self.kv_heads, self.vdim, view.page_size, self.pb if self.head_bias else None,
                                   self.scale, self.window, gate)
         return self.o(out)

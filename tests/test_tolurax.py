@@ -22,7 +22,7 @@ DTYPES = ["float32", "bfloat16"]
 MODELS = {"X": (M.CONFIG_X, 11, False, 8), "Y": (M.CONFIG_Y, 12, False, 16), "Z": (M.CONFIG_Z, 13, False, 4),
           "X-sharp": (M.CONFIG_X, 14, True, 16), "Y-sharp": (M.CONFIG_Y, 15, True, 8),
           "delta": (M.ONLY_DELTA, 16, False, 8), "left": (M.ONLY_LEFT, 17, True, 8), "right": (M.ONLY_RIGHT, 18, False, 8),
-          "filter-ffn": (M.ONLY_FILTER_FFN, 19, False, 8)}
+          "filter-ffn": (M.ONLY_FILTER_FFN, 19, False, 8), "W-sharp": (M.CONFIG_W, 20, True, 16)}
 LENGTHS = (40, 70, 33, 58, 50, 64, 21)
 # bfloat16 engine against the float64 plain model, relative rms of the logits: what rounding alone gives on these
 # models stays below a third of this; a lost key, state or filter input is far above it on the sharp models.
@@ -95,7 +95,7 @@ def test_every_way_of_cutting(folders, name, dtype, device):
 
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["X", "Y-sharp", "Z"])
+@pytest.mark.parametrize("name", ["X", "Y-sharp", "Z", "W-sharp"])
 def test_mixed_batches_in_a_small_pool(folders, name, dtype, device):
     """Unequal requests side by side (portions beside single tokens, requests left out of steps) against each alone;
     three slots and a pool of the trace's peak, so that pages and slots are given back and used again."""
@@ -129,40 +129,43 @@ def test_float32_does_not_depend_on_the_cut(folders, device):
                 assert H.rel_rms(row, whole[key]) < 1e-5
 
 
-def _needle_model(root, window, page):
-    """One parallel layer whose attention alone reaches the stream (no rotation, no filter, memory scaled by 0), with
-    head biases of -14: a key counts only where its score is far above the others'. Returns the folder and a pair of
-    token ids (query token, key token) whose score stands out, with a filler token that matches nothing."""
+def _needle_model(root, window, page, dim=16):
+    """One parallel layer whose attention alone reaches the stream (no rotation, no filter, memory scaled by 0). A
+    pair of token ids (query token, key token) whose score is the largest of all, and a filler token whose scores
+    with them and with itself are lowest; the head biases are then set so that the pair's weight is sigmoid(3) and
+    every other weight in the test's prompts below sigmoid(-4). Returns the folder and the three ids."""
     cfg = {"architecture": "Tolurax", "width": 32, "vocab": 40, "norm": {"eps": 1e-6},
-           "layers": [M.parallel(M.left(2, 1, 16, 16, window, 1.0), 1, 8, 1.0, 0.0)]}
+           "layers": [M.parallel(M.left(2, 1, dim, dim, window, 16.0 / dim), 1, 8, 1.0, 0.0)]}
+    found = {}
 
     def edit(t):
-        t["l0.mix.left.pb"] = torch.full((2,), -14.0).bfloat16()
-        t["l0.mix.left.q.norm"] = (t["l0.mix.left.q.norm"].float() * 1.6).bfloat16()
-        t["l0.mix.left.k.norm"] = (t["l0.mix.left.k.norm"].float() * 1.6).bfloat16()
+        for name in ("l0.mix.left.q.norm", "l0.mix.left.k.norm"):
+            t[name] = (t[name].float() * 1.6).bfloat16()
+        get = lambda n: t[n].double()                          # noqa: E731
+        h = M.plain.layer_norm(get("embed"), get("l0.norm1"), 1e-6)       # every token's mixer input
+        q = (h @ get("l0.mix.left.q").T).view(-1, 2, dim)
+        k = (h @ get("l0.mix.left.k").T).view(-1, 1, dim)
+        q = M.plain.rms_div(q, 1e-6) * get("l0.mix.left.q.norm")
+        k = M.plain.rms_div(k, 1e-6) * get("l0.mix.left.k.norm")
+        score = torch.einsum("ahd,bd->abh", q, k[:, 0]).amax(-1) * 16.0 / dim    # [query token, key token]
+        a, b = divmod(int(score.argmax()), score.shape[1])
+        others = torch.stack((score[a], score[:, b], score.diagonal())).amax(0)
+        filler = int(others.argmin())
+        assert score[a, b] - others[filler] > 7, "the needle does not stand out"
+        t["l0.mix.left.pb"] = torch.full((2,), 3.0 - float(score[a, b])).bfloat16()
+        found.update(a=a, b=b, filler=filler)
     folder = M.make_folder(root, cfg, 77, sharp=False, edit=edit)
-    p, tensors = M.PlainTolurax(folder), None
-    get = lambda n: p.tensors[n].double()                      # noqa: E731
-    h = M.plain.layer_norm(get("embed"), get("l0.norm1"), 1e-6)           # every token's mixer input
-    q = (h @ get("l0.mix.left.q").T).view(-1, 2, 16)
-    k = (h @ get("l0.mix.left.k").T).view(-1, 1, 16)
-    q = M.plain.rms_div(q, 1e-6) * get("l0.mix.left.q.norm")
-    k = M.plain.rms_div(k, 1e-6) * get("l0.mix.left.k.norm")
-    score = torch.einsum("ahd,bd->abh", q, k[:, 0]).amax(-1)              # [query token, key token]
-    a, b = divmod(int(score.argmax()), score.shape[1])
-    filler = int((score[a] + score[:, b] + score.diagonal()).argmin())
-    assert score[a, b] > 14 and score[a, filler] < 8 and score[filler, b] < 8, "the needle does not stand out"
-    return folder, a, b, filler
+    return folder, found["a"], found["b"], found["filler"]
 
 
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("window,page", [(21, 8), (16, 16), (40, 16)])
-def test_a_key_just_inside_and_just_outside_the_window(tmp_path, window, page, dtype, device):
+@pytest.mark.parametrize("window,page,dim", [(21, 8, 16), (16, 16, 16), (35, 16, 64), (70, 32, 128)])
+def test_a_key_just_inside_and_just_outside_the_window(tmp_path, window, page, dim, dtype, device):
     """One key whose score stands out, `window - 1` and `window` tokens behind the query, the key on either side of a
     page border: the plain model says the logits differ widely between the two, and the engine follows it both in a
     prompt and when the query is decoded alone."""
-    folder, a, b, filler = _needle_model(tmp_path / "needle", window, page)
+    folder, a, b, filler = _needle_model(tmp_path / "needle", window, page, dim)
     plain = M.PlainTolurax(folder)
     for key_at in (page - 1, page, 2 * page + 3):
         inside = [filler] * key_at + [b] + [filler] * (window - 2) + [a, filler]
@@ -171,7 +174,7 @@ def test_a_key_just_inside_and_just_outside_the_window(tmp_path, window, page, d
         gap = H.rel_rms(plain.logits(inside)[qi], plain.logits(outside)[qo])
         assert gap > 0.3, f"the test's key does not show: {gap}"
         for ids, at, what in ((inside, qi, "inside"), (outside, qo, "outside")):
-            rep = _replayer(folder, device, dtype, page, cache_tokens=-(-len(ids) // page) * page, max_model_len=128)
+            rep = _replayer(folder, device, dtype, page, cache_tokens=-(-len(ids) // page) * page, max_model_len=192)
             got = H.run_trace(rep, H.trace_whole({"p": ids}))
             _check(folder, dtype, {"p": ids}, got, f"window {window} key at {key_at} {what}, prompt")
             got = H.run_trace(rep, H.trace_decode_tail("p", ids, len(ids) - at + 2))

@@ -49,6 +49,12 @@ CONFIG_Y = {"architecture": "Tolurax", "width": 96, "vocab": 200, "norm": {"eps"
 CONFIG_Z = {"architecture": "Tolurax", "width": 32, "vocab": 50, "norm": {"eps": 1e-6},
             "loop": {"start": 0, "stop": 2, "times": 1},
             "layers": [parallel(left(1, 1, 8, 8, 1, 1.0), 1, 8, 1.0, 1.0, ff=32), delta(1, 1, 8, 8, 1)]}
+# W: heads of 64 with keys and values of one width (what the matrix-core prompt kernel serves), a window of 50 over
+# pages of 16, grouped heads, part of the head rotated.
+CONFIG_W = {"architecture": "Tolurax", "width": 96, "vocab": 120, "norm": {"eps": 1e-6}, "canon": {"taps": 3},
+            "logit_softcap": 20.0,
+            "layers": [parallel(left(4, 2, 64, 64, 50, 0.125, {"dims": 32, "base": 10000.0}), 2, 32, ff=128),
+                       delta(2, 1, 64, 64, 4)]}
 # One mechanism at a time.
 ONLY_DELTA = {"architecture": "Tolurax", "width": 48, "vocab": 90, "norm": {"eps": 1e-6},
               "layers": [delta(4, 1, 24, 12, 4), delta(3, 3, 16, 16, 2)]}
