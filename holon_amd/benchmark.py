@@ -20,6 +20,11 @@ The engine is one process on one GPU; for --gpus > 1 a line says so and the exit
 --workload runs a whole job through the engine instead and prints its own line: `mixed` is 32 requests of 128 to 4,096
 prompt tokens at the Qwen3-32B shape, portions of 512 tokens beside decode rows, 256 greedy tokens each; `long` is 8
 prompts of 32,768 tokens at the Qwen3-4B shape, 512 tokens each at temperature 0.7.
+
+--workload tolurax measures the Tolurax design beside Qwen3 at equal sizes (width, layers, heads, head size,
+feed-forward, vocabulary; random weights): a 2,048-token prompt and decode at batch 8 near a context of 2,048, at two
+sizes (`--sizes`), one line with both models' figures and the bytes a decode step must read. `--only` runs one model
+(for a profiler).
 """
 from __future__ import annotations
 
@@ -95,6 +100,110 @@ def workload(name: str, layers: int | None, dtype: str, products: str = "timed")
     return 0
 
 
+DESIGN_SIZES = {     # width, layers, heads, kv heads, head size, feed-forward, vocabulary
+    "2k": dict(width=2048, layers=8, heads=16, kv_heads=4, dim=128, ff=8192, vocab=32768),
+    "4k": dict(width=4096, layers=4, heads=32, kv_heads=8, dim=128, ff=12288, vocab=32768)}
+
+
+def tolurax_config(z: dict, window: int = 1024) -> dict:
+    """A Tolurax model of a size's layers: three parallel layers (windowed sigmoid attention with the size's heads
+    beside a decayed memory of heads of 64 over the same width) to every delta layer, a feed-forward in each."""
+    def layer(i: int) -> dict:
+        mlp = {"kind": "dense", "ff": z["ff"]}
+        if i % 4 == 3:
+            return {"type": "delta", "mlp": mlp, "mixer": {"heads": z["heads"], "kv_heads": z["heads"], "dim": z["dim"],
+                                                          "vdim": z["dim"], "conv": 4}}
+        left = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["dim"],
+                "mask": {"size": window}, "scale": z["dim"] ** -0.5,
+                "rot": {"dims": z["dim"], "base": 10000.0,
+                        "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}}
+        right = {"heads": z["width"] // 64, "dim": 64, "rank": 64}
+        return {"type": "parallel", "mlp": mlp, "mixer": {"left": left, "right": right, "left_scale": 1.0,
+                                                          "right_scale": 1.0}}
+    return {"architecture": "Tolurax", "width": z["width"], "vocab": z["vocab"], "norm": {"eps": 1e-6},
+            "canon": {"taps": 3}, "logit_softcap": 30.0, "layers": [layer(i) for i in range(z["layers"])]}
+
+
+def qwen3_config(z: dict) -> dict:
+    return {"architectures": ["Qwen3ForCausalLM"], "num_hidden_layers": z["layers"], "hidden_size": z["width"],
+            "num_attention_heads": z["heads"], "num_key_value_heads": z["kv_heads"], "head_dim": z["dim"],
+            "intermediate_size": z["ff"], "vocab_size": z["vocab"], "rope_theta": 1e6, "rms_norm_eps": 1e-6,
+            "tie_word_embeddings": False, "max_position_embeddings": 8192}
+
+
+def design(a) -> int:
+    """Tolurax beside Qwen3 at equal sizes: prompt and decode throughput, one line."""
+    import gc
+
+    import torch
+
+    from .config import EngineConfig, SamplingParams
+    from .engine.engine import Engine
+    prompt, context, batch = 2048, 2048, 8
+    g = torch.Generator().manual_seed(0)
+    greedy = lambda n: SamplingParams(temperature=0.0, max_tokens=n, ignore_eos=True)      # noqa: E731
+    out: dict = {}
+    for size in a.sizes.split(","):
+        z = DESIGN_SIZES[size]
+        for name, cfg_json in (("tolurax", tolurax_config(z)), ("qwen3", qwen3_config(z))):
+            if a.only and a.only != name:
+                continue
+            engine = Engine.from_random(cfg_json, seed=0, cfg=EngineConfig(
+                model=f"random:{name}-{size}", device="cuda:0", dtype=a.dtype, page_size=16, max_seqs=batch,
+                max_model_len=context + 64, max_step_tokens=4096, cache_tokens=batch * (context + 64),
+                graphs=not a.no_graphs, products=a.products, prefix_cache=False))
+            item = 2 if a.dtype == "bfloat16" else 4
+            weights = sum(getattr(o, n).numel() * getattr(o, n).element_size()
+                          for path, o, n, _ in engine.model.named_params() if not path.startswith("embed."))
+            state = engine.cache.nbytes() // (batch + 1) if name == "tolurax" else 0   # slot state (read and written)
+            times = []
+            for _ in range(3):
+                engine.add(torch.randint(0, z["vocab"], (prompt,), generator=g).tolist(), greedy(1))
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                while engine.has_work():
+                    engine.step()
+                engine.drain()
+                torch.cuda.synchronize()
+                times.append((time.perf_counter() - t0) * 1e3)
+            start = context - a.steps - a.warmup - 3
+            for _ in range(batch):
+                engine.add(torch.randint(0, z["vocab"], (start,), generator=g).tolist(), greedy(a.steps + a.warmup + 3))
+            while engine.sched.waiting:
+                engine.step()
+            for _ in range(a.warmup):
+                engine.step()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(a.steps):
+                engine.step()
+            torch.cuda.synchronize()
+            ms = (time.perf_counter() - t0) * 1e3 / a.steps
+            while engine.has_work():
+                engine.step()
+            kv = 0 if name == "tolurax" else z["layers"] * 2 * z["kv_heads"] * z["dim"] * item * batch * context
+            if name == "tolurax":           # the window's keys and values of the parallel layers
+                kv = sum(2 * z["kv_heads"] * z["dim"] * item * batch * min(context, 1024)
+                         for layer in cfg_json["layers"] if layer["type"] == "parallel")
+            step_gb = (weights + kv + 2 * state * batch) / 1e9
+            out.setdefault(size, {})[name] = {
+                "prefill_tokens_per_s": round(prompt / (min(times) * 1e-3), 1), "prefill_ms": round(min(times), 3),
+                "prefill_ms_median": round(sorted(times)[1], 3), "decode_tokens_per_s": round(batch / (ms * 1e-3), 1),
+                "decode_ms_per_step": round(ms, 4), "decode_step_gb": round(step_gb, 3),
+                "decode_frac_of_hbm": round(step_gb / (ms * 1e-3) / HBM_GBS, 4),
+                "graphs": engine.runner.use_graphs}
+            engine.close()
+            del engine
+            gc.collect()
+            torch.cuda.empty_cache()
+    print(json.dumps({"metric": "Tolurax beside Qwen3 at equal sizes: 2,048-token prompt, decode at batch 8 near context 2,048",
+                      "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+                      "dtype": "bf16" if a.dtype == "bfloat16" else "fp32",
+                      "data": "synthetic (random weights, uniform random token ids)",
+                      "sizes": {k: DESIGN_SIZES[k] for k in out}, "results": out}), flush=True)
+    return 0
+
+
 def main(argv: list[str] | None = None) -> int:
     ap = argparse.ArgumentParser(prog="bench", description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
@@ -109,7 +218,9 @@ def main(argv: list[str] | None = None) -> int:
     ap.add_argument("--context", type=int, default=CONTEXT, help="the context the timed decode steps end at")
     ap.add_argument("--prompt", type=int, default=PROMPT, help="tokens of the timed prompt")
     ap.add_argument("--no-graphs", action="store_true")
-    ap.add_argument("--workload", choices=("decode", "mixed", "long"), default="decode")
+    ap.add_argument("--workload", choices=("decode", "mixed", "long", "tolurax"), default="decode")
+    ap.add_argument("--sizes", default="2k,4k", help="--workload tolurax: which of its sizes (2k, 4k) to run")
+    ap.add_argument("--only", choices=("tolurax", "qwen3"), default=None, help="--workload tolurax: one model only")
     ap.add_argument("--products", choices=("own", "vendor", "timed"), default="timed",
                     help="EngineConfig.products: which kernel products of 17 to 1,024 rows take (reported in the line)")
     a = ap.parse_args(argv)
@@ -120,6 +231,8 @@ def main(argv: list[str] | None = None) -> int:
         from .kernels import build as kernel_build
         if kernel_build.find_library() is None:
             kernel_build.build()
+        if a.workload == "tolurax":
+            return design(a)
         return workload(a.workload, None if "--layers" not in (argv or sys.argv) else a.layers, a.dtype, a.products)
 
     import torch

@@ -209,8 +209,8 @@ int holon_gated_out(const float* o, const void* gate, const void* weight, void* 
 int holon_shift_mix(const void* x, const void* mu, void* state, void* y, const int32_t* slots, const int32_t* starts,
                     const int32_t* query_start, const int32_t* token_row, int tokens, int rows, int width, int mixes,
                     int state_slots, int dtype, void* stream);
-// y [T, C] = exp(-exp(tanh(a [T, R]) w2 [C, R]^T + w0 [C])), float32.
-int holon_decay_lora(const float* a, const void* w2, const float* w0, float* y, int tokens, int channels, int rank,
+// y [T, C] = exp(-exp(tanh(a [T, R]) w2^T + w0 [C])), float32; w2 comes transposed, w2t [R, C].
+int holon_decay_lora(const float* a, const void* w2t, const float* w0, float* y, int tokens, int channels, int rank,
                      int dtype, void* stream);
 
 // -- windowed sigmoid attention (sigmoid_attention.hip); a page is keys [Hkv, P, D] then values [Hkv, V, P] ---------------

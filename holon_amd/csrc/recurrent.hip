@@ -107,8 +107,13 @@ __device__ __forceinline__ float quad_sum(float v) {
 
 constexpr int SCAN_COLS = 16;      // value columns a wave owns; four lanes a column, each a quarter of the key rows
 
+// Tokens a wave stages at a time: their operands travel from memory to LDS as one batch of loads while the batch before
+// is worked through, so that a token's arithmetic never waits for memory (one token at a time, a step took as long as
+// a load: 0.9 us). About a thousand values per operand and batch.
+template <int KD> struct ScanChunk { static constexpr int kTokens = KD <= 64 ? 16 : KD <= 128 ? 8 : 4; };
+
 // Per (row, head): S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q. Lane 4 c + p owns rows
-// p KD/4 .. (p + 1) KD/4 - 1 of column c of S. The next token's operands are asked for before this token's arithmetic.
+// p KD/4 .. (p + 1) KD/4 - 1 of column c of S.
 template <int KD, typename T>
 __global__ void __launch_bounds__(WAVE) delta_scan_kernel(const float* __restrict__ qn, const float* __restrict__ kn,
                                                           const T* __restrict__ qkv, int qkv_stride, int v_offset,
@@ -118,10 +123,12 @@ __global__ void __launch_bounds__(WAVE) delta_scan_kernel(const float* __restric
                                                           const int32_t* __restrict__ starts,
                                                           const int32_t* __restrict__ query_start, int heads,
                                                           int kv_heads, int dim, int vdim) {
-  constexpr int KQ = KD / 4, PER = (KD + WAVE - 1) / WAVE;
-  __shared__ float ks[KD], qs[KD];
+  constexpr int KQ = KD / 4, TC = ScanChunk<KD>::kTokens, N = TC * KD, PER = (N + WAVE - 1) / WAVE;
+  constexpr int VPER = (TC * SCAN_COLS + WAVE - 1) / WAVE;
+  __shared__ __attribute__((aligned(16))) float ks[2][N], qs[2][N];
+  __shared__ float vs[2][TC * SCAN_COLS], gs[2][TC], bs[2][TC];
   const int b = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-  const int part = lane % 4, j = blockIdx.z * SCAN_COLS + lane / 4;
+  const int part = lane % 4, col = lane / 4, j = blockIdx.z * SCAN_COLS + col;
   const int hk = h / (heads / kv_heads);
   const bool active = j < vdim;
   const int lo = query_start[b], hi = query_start[b + 1];
@@ -133,44 +140,69 @@ __global__ void __launch_bounds__(WAVE) delta_scan_kernel(const float* __restric
     const int row = part * KQ + i;
     S[i] = (carried && active && row < dim) ? held[(int64_t)row * vdim + j] : 0.f;
   }
-  float nk[PER], nq[PER], ng = 0.f, nb = 0.f, nv = 0.f;
-  auto ask = [&](int t) {
+  float nk[PER], nq[PER], nv[VPER], ng = 1.f, nb = 0.f;
+  auto ask = [&](int t0) {
 #pragma unroll
     for (int e = 0; e < PER; ++e) {
-      const int i = lane + e * WAVE;
-      nk[e] = i < dim ? kn[((int64_t)t * kv_heads + hk) * dim + i] : 0.f;
-      nq[e] = i < dim ? qn[((int64_t)t * kv_heads + hk) * dim + i] : 0.f;
+      const int idx = lane + e * WAVE, tt = idx / KD, i = idx - tt * KD;
+      const bool ok = idx < N && t0 + tt < hi && i < dim;
+      const int64_t at = ((int64_t)(t0 + tt) * kv_heads + hk) * dim + i;
+      nk[e] = ok ? kn[at] : 0.f;
+      nq[e] = ok ? qn[at] : 0.f;
     }
-    ng = g[(int64_t)t * heads + h];
-    nb = beta[(int64_t)t * heads + h];
-    nv = active ? Elem<T>::load(qkv[(int64_t)t * qkv_stride + v_offset + h * vdim + j]) : 0.f;
+#pragma unroll
+    for (int e = 0; e < VPER; ++e) {
+      const int idx = lane + e * WAVE, tt = idx / SCAN_COLS, jj = blockIdx.z * SCAN_COLS + idx % SCAN_COLS;
+      const bool ok = idx < TC * SCAN_COLS && t0 + tt < hi && jj < vdim;
+      nv[e] = ok ? Elem<T>::load(qkv[(int64_t)(t0 + tt) * qkv_stride + v_offset + h * vdim + jj]) : 0.f;
+    }
+    const bool ok = lane < TC && t0 + lane < hi;
+    ng = ok ? g[(int64_t)(t0 + lane) * heads + h] : 1.f;
+    nb = ok ? beta[(int64_t)(t0 + lane) * heads + h] : 0.f;
   };
-  if (lo < hi) ask(lo);
-  for (int t = lo; t < hi; ++t) {
-    __syncthreads();
+  auto put = [&](int buf) {
 #pragma unroll
     for (int e = 0; e < PER; ++e) {
-      const int i = lane + e * WAVE;
-      if (i < KD) { ks[i] = nk[e]; qs[i] = nq[e]; }
+      const int idx = lane + e * WAVE;
+      if (idx < N) { ks[buf][idx] = nk[e]; qs[buf][idx] = nq[e]; }
     }
-    const float gt = ng, bt = nb, vt = nv;
+#pragma unroll
+    for (int e = 0; e < VPER; ++e) {
+      const int idx = lane + e * WAVE;
+      if (idx < TC * SCAN_COLS) vs[buf][idx] = nv[e];
+    }
+    if (lane < TC) { gs[buf][lane] = ng; bs[buf][lane] = nb; }
+  };
+  if (lo < hi) {
+    ask(lo);
+    put(0);
+  }
+  __syncthreads();
+  for (int t0 = lo, buf = 0; t0 < hi; t0 += TC, buf ^= 1) {
+    if (t0 + TC < hi) ask(t0 + TC);
+    const int nt = min(TC, hi - t0);
+    for (int tt = 0; tt < nt; ++tt) {
+      const float gt = gs[buf][tt], bt = bs[buf][tt], vt = vs[buf][tt * SCAN_COLS + col];
+      const float* kt = &ks[buf][tt * KD + part * KQ];
+      const float* qt = &qs[buf][tt * KD + part * KQ];
+      float dot = 0.f;
+#pragma unroll
+      for (int i = 0; i < KQ; ++i) {
+        S[i] *= gt;
+        dot += S[i] * kt[i];
+      }
+      const float u = bt * (vt - quad_sum(dot));
+      float o = 0.f;
+#pragma unroll
+      for (int i = 0; i < KQ; ++i) {
+        S[i] += kt[i] * u;
+        o += S[i] * qt[i];
+      }
+      o = quad_sum(o);
+      if (active && part == 0) out[((int64_t)(t0 + tt) * heads + h) * vdim + j] = o;
+    }
+    if (t0 + TC < hi) put(buf ^ 1);
     __syncthreads();
-    if (t + 1 < hi) ask(t + 1);
-    float dot = 0.f;
-#pragma unroll
-    for (int i = 0; i < KQ; ++i) {
-      S[i] *= gt;
-      dot += S[i] * ks[part * KQ + i];
-    }
-    const float u = bt * (vt - quad_sum(dot));
-    float o = 0.f;
-#pragma unroll
-    for (int i = 0; i < KQ; ++i) {
-      S[i] += ks[part * KQ + i] * u;
-      o += S[i] * qs[part * KQ + i];
-    }
-    o = quad_sum(o);
-    if (active && part == 0) out[((int64_t)t * heads + h) * vdim + j] = o;
   }
   if (active) {
 #pragma unroll
@@ -189,10 +221,12 @@ __global__ void __launch_bounds__(WAVE) memory_scan_kernel(const T* __restrict__
                                                            float* __restrict__ out, const int32_t* __restrict__ slots,
                                                            const int32_t* __restrict__ starts,
                                                            const int32_t* __restrict__ query_start, int heads, int dim) {
-  constexpr int KQ = KD / 4, PER = (KD + WAVE - 1) / WAVE;
-  __shared__ float rs[KD], ks[KD], ws[KD], us[KD];
+  constexpr int KQ = KD / 4, TC = ScanChunk<KD>::kTokens, N = TC * KD, PER = (N + WAVE - 1) / WAVE;
+  constexpr int VPER = (TC * SCAN_COLS + WAVE - 1) / WAVE;
+  __shared__ __attribute__((aligned(16))) float rs[2][N], ks[2][N], ws[2][N], us[KD];
+  __shared__ float vs[2][TC * SCAN_COLS];
   const int b = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-  const int part = lane % 4, j = blockIdx.z * SCAN_COLS + lane / 4;
+  const int part = lane % 4, col = lane / 4, j = blockIdx.z * SCAN_COLS + col;
   const bool active = j < dim;
   const int lo = query_start[b], hi = query_start[b + 1];
   float* held = state + ((int64_t)slots[b] * heads + h) * dim * dim;
@@ -205,39 +239,62 @@ __global__ void __launch_bounds__(WAVE) memory_scan_kernel(const T* __restrict__
   }
   for (int i = lane; i < KD; i += WAVE) us[i] = i < dim ? u[h * dim + i] : 0.f;
   const int64_t width = (int64_t)heads * dim;
-  float nr[PER], nk[PER], nw[PER], nv = 0.f;
-  auto ask = [&](int t) {
+  float nr[PER], nk[PER], nw[PER], nv[VPER];
+  auto ask = [&](int t0) {
 #pragma unroll
     for (int e = 0; e < PER; ++e) {
-      const int i = lane + e * WAVE;
-      const int64_t at = (int64_t)t * width + h * dim + i;
-      nr[e] = i < dim ? Elem<T>::load(r[at]) : 0.f;
-      nk[e] = i < dim ? Elem<T>::load(k[at]) : 0.f;
-      nw[e] = i < dim ? w[at] : 0.f;
+      const int idx = lane + e * WAVE, tt = idx / KD, i = idx - tt * KD;
+      const bool ok = idx < N && t0 + tt < hi && i < dim;
+      const int64_t at = (int64_t)(t0 + tt) * width + h * dim + i;
+      nr[e] = ok ? Elem<T>::load(r[at]) : 0.f;
+      nk[e] = ok ? Elem<T>::load(k[at]) : 0.f;
+      nw[e] = ok ? w[at] : 0.f;
     }
-    nv = active ? Elem<T>::load(v[(int64_t)t * width + h * dim + j]) : 0.f;
+#pragma unroll
+    for (int e = 0; e < VPER; ++e) {
+      const int idx = lane + e * WAVE, tt = idx / SCAN_COLS, jj = blockIdx.z * SCAN_COLS + idx % SCAN_COLS;
+      const bool ok = idx < TC * SCAN_COLS && t0 + tt < hi && jj < dim;
+      nv[e] = ok ? Elem<T>::load(v[(int64_t)(t0 + tt) * width + h * dim + jj]) : 0.f;
+    }
   };
-  if (lo < hi) ask(lo);
-  for (int t = lo; t < hi; ++t) {
-    __syncthreads();
+  auto put = [&](int buf) {
 #pragma unroll
     for (int e = 0; e < PER; ++e) {
-      const int i = lane + e * WAVE;
-      if (i < KD) { rs[i] = nr[e]; ks[i] = nk[e]; ws[i] = nw[e]; }
+      const int idx = lane + e * WAVE;
+      if (idx < N) { rs[buf][idx] = nr[e]; ks[buf][idx] = nk[e]; ws[buf][idx] = nw[e]; }
     }
-    const float vt = nv;
-    __syncthreads();
-    if (t + 1 < hi) ask(t + 1);
-    float o = 0.f;
 #pragma unroll
-    for (int i = 0; i < KQ; ++i) {
-      const int row = part * KQ + i;
-      const float kv = ks[row] * vt;
-      o += rs[row] * (S[i] + us[row] * kv);
-      S[i] = ws[row] * S[i] + kv;
+    for (int e = 0; e < VPER; ++e) {
+      const int idx = lane + e * WAVE;
+      if (idx < TC * SCAN_COLS) vs[buf][idx] = nv[e];
     }
-    o = quad_sum(o);
-    if (active && part == 0) out[(int64_t)t * width + h * dim + j] = o;
+  };
+  if (lo < hi) {
+    ask(lo);
+    put(0);
+  }
+  __syncthreads();
+  for (int t0 = lo, buf = 0; t0 < hi; t0 += TC, buf ^= 1) {
+    if (t0 + TC < hi) ask(t0 + TC);
+    const int nt = min(TC, hi - t0);
+    for (int tt = 0; tt < nt; ++tt) {
+      const float vt = vs[buf][tt * SCAN_COLS + col];
+      const float* rt = &rs[buf][tt * KD + part * KQ];
+      const float* kt = &ks[buf][tt * KD + part * KQ];
+      const float* wt = &ws[buf][tt * KD + part * KQ];
+      const float* ut = &us[part * KQ];
+      float o = 0.f;
+#pragma unroll
+      for (int i = 0; i < KQ; ++i) {
+        const float kv = kt[i] * vt;
+        o += rt[i] * (S[i] + ut[i] * kv);
+        S[i] = wt[i] * S[i] + kv;
+      }
+      o = quad_sum(o);
+      if (active && part == 0) out[(int64_t)(t0 + tt) * width + h * dim + j] = o;
+    }
+    if (t0 + TC < hi) put(buf ^ 1);
+    __syncthreads();
   }
   if (active) {
 #pragma unroll
@@ -295,20 +352,34 @@ __global__ void shift_keep_kernel(const T* __restrict__ x, T* __restrict__ state
   state[(int64_t)slots[b] * width + c] = x[(int64_t)(query_start[b + 1] - 1) * width + c];
 }
 
-// One block a token: exp(-exp(tanh(a) w2^T + w0)), the rank's tanh values shared through LDS.
+// exp(-exp(tanh(a) w2^T + w0)): a block takes 8 tokens and 256 channels; the tokens' tanh values are shared through
+// LDS, and w2 comes transposed ([rank, channels]) so that a wave's loads are contiguous and serve all 8 tokens.
+constexpr int LORA_TOKENS = 8, LORA_MAX_RANK = 1024;
 template <typename T>
-__global__ void __launch_bounds__(256) decay_lora_kernel(const float* __restrict__ a, const T* __restrict__ w2,
-                                                         const float* __restrict__ w0, float* __restrict__ y,
+__global__ void __launch_bounds__(256) decay_lora_kernel(const float* __restrict__ a, const T* __restrict__ w2t,
+                                                         const float* __restrict__ w0, float* __restrict__ y, int tokens,
                                                          int channels, int rank) {
-  __shared__ float th[1024];
-  const int t = blockIdx.x;
-  for (int r = threadIdx.x; r < rank; r += 256) th[r] = tanhf(a[(int64_t)t * rank + r]);
-  __syncthreads();
-  for (int c = threadIdx.x; c < channels; c += 256) {
-    float acc = 0.f;
-    for (int r = 0; r < rank; ++r) acc += th[r] * Elem<T>::load(w2[(int64_t)c * rank + r]);
-    y[(int64_t)t * channels + c] = expf(-expf(acc + w0[c]));
+  __shared__ float th[LORA_TOKENS][LORA_MAX_RANK];
+  const int t0 = blockIdx.x * LORA_TOKENS;
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  for (int e = threadIdx.x; e < LORA_TOKENS * rank; e += 256) {
+    const int tt = e / rank, r = e - tt * rank;
+    th[tt][r] = t0 + tt < tokens ? tanhf(a[(int64_t)(t0 + tt) * rank + r]) : 0.f;
   }
+  __syncthreads();
+  if (c >= channels) return;
+  float acc[LORA_TOKENS];
+#pragma unroll
+  for (int tt = 0; tt < LORA_TOKENS; ++tt) acc[tt] = 0.f;
+  for (int r = 0; r < rank; ++r) {
+    const float wv = Elem<T>::load(w2t[(int64_t)r * channels + c]);
+#pragma unroll
+    for (int tt = 0; tt < LORA_TOKENS; ++tt) acc[tt] += th[tt][r] * wv;
+  }
+  const float off = w0[c];
+#pragma unroll
+  for (int tt = 0; tt < LORA_TOKENS; ++tt)
+    if (t0 + tt < tokens) y[(int64_t)(t0 + tt) * channels + c] = expf(-expf(acc[tt] + off));
 }
 
 }  // namespace
@@ -445,12 +516,15 @@ extern "C" int holon_shift_mix(const void* x, const void* mu, void* state, void*
   return 0;
 }
 
-extern "C" int holon_decay_lora(const float* a, const void* w2, const float* w0, float* y, int tokens, int channels,
+extern "C" int holon_decay_lora(const float* a, const void* w2t, const float* w0, float* y, int tokens, int channels,
                                 int rank, int dtype, void* stream) {
-  HOLON_CHECK(tokens >= 0 && channels > 0 && rank > 0 && rank <= 1024, "decay_lora: %d channels, rank %d (at most 1024)",
-              channels, rank);
+  HOLON_CHECK(tokens >= 0 && channels > 0 && rank > 0 && rank <= LORA_MAX_RANK,
+              "decay_lora: %d channels, rank %d (at most %d)", channels, rank, LORA_MAX_RANK);
   if (tokens == 0) return 0;
-  BY_DTYPE(dtype, (decay_lora_kernel<T><<<tokens, 256, 0, (hipStream_t)stream>>>(a, (const T*)w2, w0, y, channels, rank)));
+  const dim3 grid((tokens + LORA_TOKENS - 1) / LORA_TOKENS, (channels + 255) / 256);
+  HOLON_CHECK(grid.y <= 65535, "decay_lora: %d channels exceed one launch", channels);
+  BY_DTYPE(dtype, (decay_lora_kernel<T><<<grid, 256, 0, (hipStream_t)stream>>>(a, (const T*)w2t, w0, y, tokens, channels,
+                                                                               rank)));
   HOLON_LAUNCH_OK();
   return 0;
 }

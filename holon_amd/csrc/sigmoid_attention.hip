@@ -6,7 +6,8 @@
 // norms and rotates the heads of a merged q/k/v projection and stores keys and values; `sigmoid_attention` sums
 // sigmoid(q . k * scale + bias) * v over the keys a query sees. Nothing is normalised over keys, so there is no running
 // maximum and no rescaling: a query's result is a plain sum, taken over its keys from the oldest visible one on, in
-// tiles of 64, an order that the query's position alone decides. Scores, weights and sums are float32.
+// tiles of 64 dealt to four waves in turn, an order that the query's position alone decides. Scores, weights and sums
+// are float32.
 #include "common.h"
 #include "holon_hip.h"
 
@@ -74,9 +75,11 @@ __global__ void __launch_bounds__(256) head_prepare_kernel(const T* __restrict__
     dst[d] = Elem<T>::store(Elem<T>::load(src[d]) * r * (w ? Elem<T>::load(w[d]) : 1.f));
 }
 
-// The general kernel (any dtype and sizes; the decode rows of every step): one wave per (token, head), four heads of
-// a token per block. A lane takes one key of a tile of 64: its score over D
-// (the query comes from LDS), its weight; then the lanes turn to the value columns and add the tile's weighted values.
+// The general kernel (any dtype and sizes; the decode rows of every step): one block of four waves per (token, head).
+// The query's keys are walked in tiles of 64 from the oldest visible one; wave w takes tiles w, w + 4, ... A lane takes
+// one key of a tile: its score over D (the query comes from LDS) and its weight; then the lanes turn to the value
+// columns and add the tile's weighted values, each weight handed round from the lane that holds it. The four waves' sums
+// are added in wave order at the end, so the order of every sum is decided by the query's position alone.
 template <typename T, bool VEC>
 __global__ void __launch_bounds__(256) sigmoid_attention_kernel(const T* __restrict__ q, T* __restrict__ out,
                                                                 const T* __restrict__ pages,
@@ -89,20 +92,18 @@ __global__ void __launch_bounds__(256) sigmoid_attention_kernel(const T* __restr
                                                                 int kv_heads, int dim, int vdim, int page_size,
                                                                 const float* __restrict__ bias, float scale, int window,
                                                                 const T* __restrict__ gate) {
-  __shared__ float q_s[4][SIG_MAX_D];
-  __shared__ float p_s[4][WAVE];
-  __shared__ int64_t v_s[4][WAVE];
+  __shared__ float q_s[SIG_MAX_D];
+  __shared__ float sum_s[4][SIG_MAX_D];
   const int w = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
   const int t = row_ids ? query_start[row_ids[blockIdx.x]] : blockIdx.x;   // the one token of a listed row, or every token
-  const bool live = blockIdx.y * 4 + w < heads;
-  const int h = live ? blockIdx.y * 4 + w : 0;       // a spare wave walks head 0 and stores nothing: all reach the barriers
+  const int h = blockIdx.y;
   const int pos = positions[t];
   const int hk = h / (heads / kv_heads);
   const int32_t* trow = table + (int64_t)slots[token_row[t]] * table_stride;
   const int64_t page_len = (int64_t)kv_heads * page_size * (dim + vdim);
   const int64_t val_base = (int64_t)kv_heads * page_size * dim;
   const T* qp = q + ((int64_t)t * heads + h) * dim;
-  for (int d = lane; d < dim; d += WAVE) q_s[w][d] = Elem<T>::load(qp[d]);
+  for (int d = threadIdx.x; d < dim; d += 256) q_s[d] = Elem<T>::load(qp[d]);
   __syncthreads();
   const float head_bias = bias ? bias[h] : 0.f;
   const int first = window > 0 ? max(0, pos - window + 1) : 0;
@@ -111,7 +112,7 @@ __global__ void __launch_bounds__(256) sigmoid_attention_kernel(const T* __restr
   for (int i = 0; i < SIG_MAX_D / WAVE; ++i) acc[i] = 0.f;
   constexpr int V = Elem<T>::kVec;
 
-  for (int j0 = first; j0 <= pos; j0 += WAVE) {
+  for (int j0 = first + w * WAVE; j0 <= pos; j0 += 4 * WAVE) {
     const int key = j0 + lane;
     float p = 0.f;
     int64_t voff = 0;
@@ -126,38 +127,37 @@ __global__ void __launch_bounds__(256) sigmoid_attention_kernel(const T* __restr
           const uint4 raw = *reinterpret_cast<const uint4*>(kp + d);
           const T* e = reinterpret_cast<const T*>(&raw);
 #pragma unroll
-          for (int i = 0; i < V; ++i) dot += q_s[w][d + i] * Elem<T>::load(e[i]);
+          for (int i = 0; i < V; ++i) dot += q_s[d + i] * Elem<T>::load(e[i]);
         }
       } else {
-        for (int d = 0; d < dim; ++d) dot += q_s[w][d] * Elem<T>::load(kp[d]);
+        for (int d = 0; d < dim; ++d) dot += q_s[d] * Elem<T>::load(kp[d]);
       }
       p = 1.0f / (1.0f + expf(-(dot * scale + head_bias)));
     }
-    p_s[w][lane] = p;
-    v_s[w][lane] = voff;
-    __syncthreads();
     const int count = min(WAVE, pos - j0 + 1);
+    for (int j = 0; j < count; ++j) {                 // j is the same in every lane: the holder's values come by readlane
+      const float pj = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(p), j));
+      const uint32_t lo = __builtin_amdgcn_readlane((uint32_t)(voff & 0xffffffffu), j);
+      const uint32_t hi = __builtin_amdgcn_readlane((uint32_t)((uint64_t)voff >> 32), j);
+      const T* vp = pages + (int64_t)(((uint64_t)hi << 32) | lo);
 #pragma unroll
-    for (int i = 0; i < SIG_MAX_D / WAVE; ++i) {
-      const int d = lane + i * WAVE;
-      if (d < vdim) {
-        float a = acc[i];
-        for (int j = 0; j < count; ++j) a += p_s[w][j] * Elem<T>::load(pages[v_s[w][j] + (int64_t)d * page_size]);
-        acc[i] = a;
+      for (int i = 0; i < SIG_MAX_D / WAVE; ++i) {
+        const int d = lane + i * WAVE;
+        if (d < vdim) acc[i] += pj * Elem<T>::load(vp[(int64_t)d * page_size]);
       }
     }
-    __syncthreads();
   }
-  if (!live) return;
 #pragma unroll
   for (int i = 0; i < SIG_MAX_D / WAVE; ++i) {
     const int d = lane + i * WAVE;
-    if (d < vdim) {
-      const int64_t at = ((int64_t)t * heads + h) * vdim + d;
-      float o = acc[i];
-      if (gate) o *= 1.0f / (1.0f + expf(-Elem<T>::load(gate[at])));
-      out[at] = Elem<T>::store(o);
-    }
+    if (d < vdim) sum_s[w][d] = acc[i];
+  }
+  __syncthreads();
+  for (int d = threadIdx.x; d < vdim; d += 256) {
+    const int64_t at = ((int64_t)t * heads + h) * vdim + d;
+    float o = ((sum_s[0][d] + sum_s[1][d]) + sum_s[2][d]) + sum_s[3][d];
+    if (gate) o *= 1.0f / (1.0f + expf(-Elem<T>::load(gate[at])));
+    out[at] = Elem<T>::store(o);
   }
 }
 }  // namespace
@@ -203,7 +203,8 @@ extern "C" int holon_sigmoid_attention(const void* q, void* out, const void* pag
   HOLON_CHECK(page_size > 0 && num_pages > 0 && window >= 0 && table_stride > 0, "sigmoid_attention: bad page geometry");
   HOLON_CHECK(row_ids == nullptr || query_start != nullptr, "sigmoid_attention: listed rows need query_start");
   if (tokens == 0) return 0;        // (with row_ids: `tokens` is the number of listed rows)
-  const dim3 grid(tokens, (heads + 3) / 4);
+  HOLON_CHECK(heads <= 65535, "sigmoid_attention: %d heads exceed one launch", heads);
+  const dim3 grid(tokens, heads);
   hipStream_t s = (hipStream_t)stream;
   const int vec = dtype == HOLON_F32 ? 4 : 8;
   const bool aligned = dim % vec == 0 && ((int64_t)vdim * page_size) % vec == 0 && (uintptr_t)pages % 16 == 0;

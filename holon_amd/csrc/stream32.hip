@@ -29,7 +29,9 @@ __global__ void widen_kernel(const void* __restrict__ x, float* __restrict__ y, 
 }
 
 // One block a row: x += s1 d1 + s2 d2 (either may be absent); then, with a weight, y = (x - mean) / sqrt(var + eps) * w
-// with the variance taken about the mean in a second pass over the row.
+// with the variance taken about the mean in a second pass over the row. REGS: the row (up to 256 * REGS values) stays in
+// registers between the passes; 0: it is read back from memory (a thread reads what it wrote itself).
+template <int REGS>
 __global__ void __launch_bounds__(256) stream_norm_kernel(float* __restrict__ x32, const void* __restrict__ d1, float s1,
                                                           int dt1, const void* __restrict__ d2, float s2, int dt2,
                                                           const void* __restrict__ weight, void* __restrict__ y, int dim,
@@ -38,23 +40,50 @@ __global__ void __launch_bounds__(256) stream_norm_kernel(float* __restrict__ x3
   const int64_t base = (int64_t)blockIdx.x * dim;
   float* x = x32 + base;
   float sum = 0.f;
-  for (int i = threadIdx.x; i < dim; i += 256) {
+  float held[REGS > 0 ? REGS : 1];
+  auto updated = [&](int i) {
     float v = x[i];
     if (d1) v += s1 * load_as(d1, base + i, dt1);
     if (d2) v += s2 * load_as(d2, base + i, dt2);
     if (d1 || d2) x[i] = v;
-    sum += v;
+    return v;
+  };
+  if constexpr (REGS > 0) {
+#pragma unroll
+    for (int e = 0; e < REGS; ++e) {
+      const int i = threadIdx.x + e * 256;
+      held[e] = i < dim ? updated(i) : 0.f;
+      sum += held[e];
+    }
+  } else {
+    for (int i = threadIdx.x; i < dim; i += 256) sum += updated(i);
   }
   if (!weight) return;
   const float mean = block_sum_256(sum, part) / (float)dim;
   float sq = 0.f;
-  for (int i = threadIdx.x; i < dim; i += 256) {     // a thread reads back what it wrote itself
-    const float d = x[i] - mean;
-    sq += d * d;
+  if constexpr (REGS > 0) {
+#pragma unroll
+    for (int e = 0; e < REGS; ++e) {
+      const float d = threadIdx.x + e * 256 < dim ? held[e] - mean : 0.f;
+      sq += d * d;
+    }
+  } else {
+    for (int i = threadIdx.x; i < dim; i += 256) {
+      const float d = x[i] - mean;
+      sq += d * d;
+    }
   }
   const float var = block_sum_256(sq, part) / (float)dim;
   const float r = 1.0f / sqrtf(var + eps);
-  for (int i = threadIdx.x; i < dim; i += 256) store_as(y, base + i, dt_out, (x[i] - mean) * r * load_as(weight, i, dt_out));
+  if constexpr (REGS > 0) {
+#pragma unroll
+    for (int e = 0; e < REGS; ++e) {
+      const int i = threadIdx.x + e * 256;
+      if (i < dim) store_as(y, base + i, dt_out, (held[e] - mean) * r * load_as(weight, i, dt_out));
+    }
+  } else {
+    for (int i = threadIdx.x; i < dim; i += 256) store_as(y, base + i, dt_out, (x[i] - mean) * r * load_as(weight, i, dt_out));
+  }
 }
 
 __global__ void pair_rows_kernel(const float* __restrict__ x32, const void* __restrict__ origin, void* __restrict__ y,
@@ -92,8 +121,14 @@ extern "C" int holon_stream_norm(float* x32, const void* d1, float s1, int dt1, 
   HOLON_CHECK(rows <= 0x7fffffff, "stream_norm: %lld rows exceed one launch", (long long)rows);
   if (rows == 0 || (!d1 && !d2 && !weight)) return 0;
   if (!d1 && d2) { d1 = d2; s1 = s2; dt1 = dt2; d2 = nullptr; }
-  stream_norm_kernel<<<(unsigned)rows, 256, 0, (hipStream_t)stream>>>(x32, d1, s1, dt1, d2, s2, dt2, weight, y, dim, eps,
-                                                                      dt_out);
+#define NORM_LAUNCH(REGS) \
+  stream_norm_kernel<REGS><<<(unsigned)rows, 256, 0, (hipStream_t)stream>>>(x32, d1, s1, dt1, d2, s2, dt2, weight, y, dim, \
+                                                                            eps, dt_out)
+  if (dim <= 1024) NORM_LAUNCH(4);          // (the sums' order is the same in every form: a thread's values in
+  else if (dim <= 2048) NORM_LAUNCH(8);     // ascending order, then the block's)
+  else if (dim <= 4096) NORM_LAUNCH(16);
+  else NORM_LAUNCH(0);
+#undef NORM_LAUNCH
   HOLON_LAUNCH_OK();
   return 0;
 }

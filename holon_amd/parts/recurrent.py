@@ -152,20 +152,20 @@ def _shift_mix_hip(launch, x, mu, state, slots, starts, query_start, token_row, 
     return y
 
 
-def decay_lora_plain(a, w2, w0):
-    """a [T, R] float32 (the decay's first projection), w2 [C, R], w0 [C] float32 ->
-    exp(-exp(tanh(a) w2^T + w0)) [T, C] float32."""
-    return torch.exp(-torch.exp(torch.tanh(a.float()) @ w2.float().t() + w0.float()))
+def decay_lora_plain(a, w2t, w0):
+    """a [T, R] float32 (the decay's first projection), w2t [R, C] (the second one, transposed), w0 [C] float32 ->
+    exp(-exp(tanh(a) w2t + w0)) [T, C] float32."""
+    return torch.exp(-torch.exp(torch.tanh(a.float()) @ w2t.float() + w0.float()))
 
 
-def _decay_lora_hip(launch, a, w2, w0):
+def _decay_lora_hip(launch, a, w2t, w0):
     t, r = a.shape
-    c = w2.shape[0]
-    _need(a.is_cuda and a.is_contiguous() and a.dtype == torch.float32 and w2.is_contiguous() and w2.dtype in _DT
-          and w2.shape[1] == r and w0.dtype == torch.float32 and w0.shape == (c,) and r <= 1024,
+    c = w2t.shape[1]
+    _need(a.is_cuda and a.is_contiguous() and a.dtype == torch.float32 and w2t.is_contiguous() and w2t.dtype in _DT
+          and w2t.shape[0] == r and w0.dtype == torch.float32 and w0.shape == (c,) and r <= 1024,
           "decay_lora: shapes do not fit (rank at most 1024)")
     y = torch.empty((t, c), dtype=torch.float32, device=a.device)
-    launch(a.data_ptr(), w2.data_ptr(), w0.data_ptr(), y.data_ptr(), t, c, r, _DT[w2.dtype])
+    launch(a.data_ptr(), w2t.data_ptr(), w0.data_ptr(), y.data_ptr(), t, c, r, _DT[w2t.dtype])
     return y
 
 
@@ -307,7 +307,7 @@ class DecayMemory(Part):
         self.declare("w0", (heads * dim,), kind=FLOAT32, init="zero")
         self.declare("u", (heads, dim), kind=FLOAT32, init="zero")
         self.declare("norm", (heads * dim,), init="norm")
-        self.mu = None
+        self.mu = self.w2t = None
 
     def state(self):
         return [SlotState(self.prefix + "shift", (self.hidden,)),
@@ -319,9 +319,10 @@ class DecayMemory(Part):
                              f"{self.w2.shape[1]}")
         if self.mu_r is not None:
             self.mu = torch.stack([getattr(self, f"mu_{s}") for s in self.MIXES]).contiguous()
+            self.w2t = self.w2.t().contiguous()       # [rank, channels]: what the decay's kernel streams
 
     def extra_tensors(self):
-        return [self.mu] if self.mu is not None else []
+        return [self.mu, self.w2t] if self.mu is not None else []
 
     def forward(self, x: torch.Tensor, step, site) -> torch.Tensor:
         k = self.kernels
@@ -329,7 +330,7 @@ class DecayMemory(Part):
         mixes = k.shift_mix(x, self.mu, site.slot_state[self.prefix + "shift"], *rows, step.token_row, step.n_rows)
         r, kk, v, gate = (getattr(self, nm)(mixes[i]) for i, nm in enumerate(("r", "k", "v", "g")))
         lora = k.linear(mixes[4], self.w1, torch.float32)
-        decay = k.decay_lora(lora, self.w2, self.w0)
+        decay = k.decay_lora(lora, self.w2t, self.w0)
         o = k.memory_scan(r, kk, v, decay, self.u, site.slot_state[self.prefix + "S"], *rows, step.n_rows, self.heads)
         return self.o(k.gated_out(o, gate, self.norm, True, self.eps, self.build.dtype))
 
