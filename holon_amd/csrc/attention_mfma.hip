@@ -126,6 +126,24 @@ __device__ __forceinline__ bf16x8_t softmax_block(const f32x4_t& s0, const f32x4
   return pb;
 }
 
+// The same place in the loop for sigmoid weights: p = 1 / (1 + exp(-(s * scale + bias))) for every visible key, 0 for the
+// others; nothing runs along (no maximum, no sum, no rescale). The weight goes to the value product as its bfloat16
+// rounding (`hi`) and the rounding of what is left (`lo`).
+__device__ __forceinline__ void sigmoid_block(const f32x4_t& s0, const f32x4_t& s1, bool whole, int kb, int g, int qp,
+                                              int first, int key_lo, int key_hi, float scale, float bias, bf16x8_t& hi,
+                                              bf16x8_t& lo) {
+#pragma unroll
+  for (int r = 0; r < 8; ++r) {
+    const float sv = r < 4 ? s0[r] : s1[r - 4];
+    const int key = kb + 8 * g + r;
+    const bool seen = whole || (key <= qp && key >= first && key >= key_lo && key <= key_hi);
+    const float e = __builtin_amdgcn_exp2f(-(fmaf(sv, scale, bias)) * 1.4426950408889634f);
+    const float p = seen ? __builtin_amdgcn_rcpf(1.0f + e) : 0.f;
+    hi[r] = (__bf16)p;
+    lo[r] = (__bf16)(p - (float)hi[r]);
+  }
+}
+
 // One wave: NT tiles against keys [key_lo, key_hi] (inclusive, as bounded per row by causality and the window).
 // On return o[t][dsub] holds the unnormalised O^T, m[t] the running max (base-2 scaled), l[t] this lane's share of
 // the sum (to be added over the four lane groups).
@@ -136,13 +154,15 @@ __device__ __forceinline__ bf16x8_t softmax_block(const f32x4_t& s0, const f32x4
 struct Nothing {
   __device__ __forceinline__ void operator()() const {}
 };
-template <int D, int NT, typename Prepare = Nothing>
+// SIG: sigmoid weights (`sig_bias[t]`: the bias of this lane's column in tile t); m and l are then left as they are.
+template <int D, int NT, typename Prepare = Nothing, bool SIG = false>
 __device__ __forceinline__ void attn_tiles(const AttnArgs& a, const int32_t* __restrict__ trow, int hk,
                                            const bf16x8_t (&qf)[NT][D / 32], const int (&qpos)[NT],
                                            const int (&tile_last)[NT], const int (&tile_first)[NT], int key_lo,
                                            int key_hi,
                                            f32x4_t (&o)[NT][D / 16], float (&m)[NT], float (&l)[NT],
-                                           const bf16_t* fresh = nullptr, Prepare prepare = Prepare()) {
+                                           const bf16_t* fresh = nullptr, Prepare prepare = Prepare(),
+                                           const float* sig_bias = nullptr) {
   const int lane = threadIdx.x % WAVE;
   const int g = lane / 16, c = lane % 16;
   const int P = a.page_size;
@@ -220,7 +240,7 @@ __device__ __forceinline__ void attn_tiles(const AttnArgs& a, const int32_t* __r
       load_keys(kb + 32, e_next, nf0, nf1);
       lookup(kb + 64, e_after);                  // (an entry past the row's keys is clamped into the table and unused)
     }
-    bf16x8_t pb[NT];
+    bf16x8_t pb[NT], pl[NT];
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
       if (kb > tile_last[t]) continue;   // every key of the block lies after every query of the tile
@@ -234,7 +254,10 @@ __device__ __forceinline__ void attn_tiles(const AttnArgs& a, const int32_t* __r
       const int first = a.window > 0 ? qp - a.window + 1 : 0;
       const bool whole = kb + 31 <= tile_first[t] && kb >= key_lo && kb + 31 <= key_hi &&
                          (a.window <= 0 || kb >= tile_last[t] - a.window + 1);
-      pb[t] = softmax_block<D / 16>(s0, s1, whole, kb, g, qp, first, key_lo, key_hi, a.scale_log2, m[t], l[t], o[t]);
+      if constexpr (SIG)
+        sigmoid_block(s0, s1, whole, kb, g, qp, first, key_lo, key_hi, a.scale, sig_bias[t], pb[t], pl[t]);
+      else
+        pb[t] = softmax_block<D / 16>(s0, s1, whole, kb, g, qp, first, key_lo, key_hi, a.scale_log2, m[t], l[t], o[t]);
     }
 #pragma unroll
     for (int ds = 0; ds < D / 16; ++ds) {
@@ -242,6 +265,7 @@ __device__ __forceinline__ void attn_tiles(const AttnArgs& a, const int32_t* __r
       for (int t = 0; t < NT; ++t) {
         if (kb > tile_last[t]) continue;
         o[t][ds] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[ds], pb[t], o[t][ds], 0, 0, 0);
+        if constexpr (SIG) o[t][ds] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[ds], pl[t], o[t][ds], 0, 0, 0);
       }
     }
     if (more) {
@@ -1464,7 +1488,9 @@ struct NewKeyValue {
 // A block's waves take consecutive shares of the row's keys and their partials are combined through LDS in wave order
 // (waves 1.. leave theirs there, wave 0 adds them up); with one block a (row, kv head) the block writes the result
 // itself and no merge kernel follows.
-template <int D, bool FUSED>
+// SIG: sigmoid weights (see AttnArgs): the waves' partials are plain sums (their maxima stay 0, so the combination above
+// adds them as they are), one block a (row, kv head) writes the result, multiplied by the gate's sigmoid if one is given.
+template <int D, bool FUSED, bool SIG = false>
 __global__ void __launch_bounds__(512) attn_decode_kernel(AttnArgs a, FusedArgs f) {
   extern __shared__ __attribute__((aligned(16))) float red[];   // [waves - 1][16 D values, 16 maxima, 16 sums]
   __shared__ __attribute__((aligned(16))) bf16_t fresh_lds[FUSED ? 2 * D : 8];
@@ -1491,7 +1517,7 @@ __global__ void __launch_bounds__(512) attn_decode_kernel(AttnArgs a, FusedArgs 
   const bool empty = n <= 0 || key_lo > key_hi;           // (uniform over the wave) a partial that weighs nothing
   const bool writer = FUSED && !empty && key_hi == qp_row;   // its keys end with the row's new token
   f32x4_t o[1][D / 16];
-  float m[1] = {-INFINITY}, l[1] = {0.f};
+  float m[1] = {SIG ? 0.f : -INFINITY}, l[1] = {0.f};
 #pragma unroll
   for (int ds = 0; ds < D / 16; ++ds) o[0][ds] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   NewKeyValue<D> fresh;
@@ -1582,8 +1608,9 @@ __global__ void __launch_bounds__(512) attn_decode_kernel(AttnArgs a, FusedArgs 
       }
     };
     int qpos[1] = {rr.valid ? qp_row : -1}, tile_last[1] = {qp_row}, tile_first[1] = {qp_row};
-    attn_tiles<D, 1>(a, trow, hk, qf, qpos, tile_last, tile_first, max(key_lo, first), key_hi, o, m, l,
-                     writer ? fresh_lds : nullptr, make_queries);
+    const float sig_bias[1] = {SIG && rr.valid && a.head_bias ? a.head_bias[rr.head] : 0.f};
+    attn_tiles<D, 1, decltype(make_queries), SIG>(a, trow, hk, qf, qpos, tile_last, tile_first, max(key_lo, first),
+                                                  key_hi, o, m, l, writer ? fresh_lds : nullptr, make_queries, sig_bias);
   }
   float lt = l[0];
   lt += __shfl_xor(lt, 16, WAVE);
@@ -1614,15 +1641,24 @@ __global__ void __launch_bounds__(512) attn_decode_kernel(AttnArgs a, FusedArgs 
   }
   if (wave == 0 && rr.valid) {
     if (a.out_splits == 1) {             // the row's whole result: normalised and rounded here
-      const float inv = lt > 0.f ? 1.0f / lt : 0.f;
+      const float inv = SIG ? 1.0f : (lt > 0.f ? 1.0f / lt : 0.f);
       bf16_t* op = a.out + ((int64_t)rr.token * a.heads + rr.head) * D + 4 * g;
+      const bf16_t* gp = SIG && a.gate ? a.gate + ((int64_t)rr.token * a.heads + rr.head) * D + 4 * g : nullptr;
 #pragma unroll
       for (int ds = 0; ds < D / 16; ++ds) {
+        float gs[4] = {1.f, 1.f, 1.f, 1.f};
+        if (SIG && gp) {
+          const ushort4 gv = *reinterpret_cast<const ushort4*>(gp + ds * 16);
+          gs[0] = 1.0f / (1.0f + __expf(-bf16_to_float(gv.x)));
+          gs[1] = 1.0f / (1.0f + __expf(-bf16_to_float(gv.y)));
+          gs[2] = 1.0f / (1.0f + __expf(-bf16_to_float(gv.z)));
+          gs[3] = 1.0f / (1.0f + __expf(-bf16_to_float(gv.w)));
+        }
         ushort4 w;
-        w.x = float_to_bf16(o[0][ds][0] * inv);
-        w.y = float_to_bf16(o[0][ds][1] * inv);
-        w.z = float_to_bf16(o[0][ds][2] * inv);
-        w.w = float_to_bf16(o[0][ds][3] * inv);
+        w.x = float_to_bf16(o[0][ds][0] * inv * gs[0]);
+        w.y = float_to_bf16(o[0][ds][1] * inv * gs[1]);
+        w.z = float_to_bf16(o[0][ds][2] * inv * gs[2]);
+        w.w = float_to_bf16(o[0][ds][3] * inv * gs[3]);
         *reinterpret_cast<ushort4*>(op + ds * 16) = w;
       }
     } else {
@@ -1835,6 +1871,38 @@ extern "C" int holon_sigmoid_attention_prefill_bf16(const void* q, void* out, co
               max_query);
   if (head_dim == 64) attn_prefill_wide_kernel<64, true><<<grid, 256, 0, (hipStream_t)stream>>>(a);
   else attn_prefill_wide_kernel<128, true><<<grid, 256, 0, (hipStream_t)stream>>>(a);
+  HOLON_LAUNCH_OK();
+  return 0;
+}
+
+// Decode rows of the same: one block a (row, kv head), the window's keys split over its waves (up to 8).
+extern "C" int holon_sigmoid_attention_decode_bf16(const void* q, void* out, const void* pages, const int32_t* table,
+                                                   int table_stride, const int32_t* slots, const int32_t* lens,
+                                                   const int32_t* query_start, const int32_t* row_ids, int n_rows,
+                                                   int max_len, int heads, int kv_heads, int head_dim, int page_size,
+                                                   float scale, int window, const float* head_bias, const void* gate,
+                                                   int rows_in_order, void* stream) {
+  HOLON_CHECK((head_dim == 64 || head_dim == 128) && mfma_serves(head_dim, page_size),
+              "sigmoid attention (matrix cores): head_dim %d / page %d not served", head_dim, page_size);
+  HOLON_CHECK(heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && window >= 0 && table_stride > 0 && max_len >= 0,
+              "sigmoid attention: bad sizes");
+  if (n_rows <= 0) return 0;
+  const int span = window > 0 ? (window < max_len ? window + 31 : max_len) : max_len;
+  int waves = (span + 127) / 128;                       // about 128 keys a wave
+  waves = waves < 1 ? 1 : (waves > 8 ? 8 : waves);
+  AttnArgs a{};
+  a.q = (const bf16_t*)q; a.out = (bf16_t*)out; a.pages = (const bf16_t*)pages; a.table = table;
+  a.table_stride = table_stride; a.slots = slots; a.lens = lens; a.qstart = query_start; a.row_ids = row_ids;
+  a.heads = heads; a.kv_heads = kv_heads; a.page_size = page_size; a.window = window;
+  a.scale = scale; a.head_bias = head_bias; a.gate = (const bf16_t*)gate;
+  a.splits = waves; a.out_splits = 1; a.rows_in_order = rows_in_order;
+  const TileMap tm = tile_map(heads / kv_heads);
+  dim3 grid(1, kv_heads * tm.head_blocks, n_rows);
+  HOLON_CHECK(grid.y <= 65535 && grid.z <= 65535, "sigmoid attention: %d rows exceed one launch", n_rows);
+  const size_t lds = (size_t)(waves - 1) * (16 * head_dim + 32) * sizeof(float);
+  const FusedArgs none{};
+  if (head_dim == 64) attn_decode_kernel<64, false, true><<<grid, waves * WAVE, lds, (hipStream_t)stream>>>(a, none);
+  else attn_decode_kernel<128, false, true><<<grid, waves * WAVE, lds, (hipStream_t)stream>>>(a, none);
   HOLON_LAUNCH_OK();
   return 0;
 }

@@ -229,6 +229,12 @@ int holon_sigmoid_attention_prefill_bf16(const void* q, void* out, const void* p
                                          const int32_t* query_start, const int32_t* row_ids, int n_rows, int max_query,
                                          int max_len, int heads, int kv_heads, int head_dim, int page_size, float scale,
                                          int window, const float* head_bias, const void* gate, void* stream);
+// The decode rows (one token each) on the matrix cores, the same sizes.
+int holon_sigmoid_attention_decode_bf16(const void* q, void* out, const void* pages, const int32_t* table,
+                                        int table_stride, const int32_t* slots, const int32_t* lens,
+                                        const int32_t* query_start, const int32_t* row_ids, int n_rows, int max_len,
+                                        int heads, int kv_heads, int head_dim, int page_size, float scale, int window,
+                                        const float* head_bias, const void* gate, int rows_in_order, void* stream);
 
 #ifdef __cplusplus
 }

@@ -4,9 +4,9 @@ i - window + 1 .. i (window 0: all before it). Scores and weights are float32.
 
 Keys and values may differ in width. One page of one site is `[Hkv, P, D]` keys (a token's key is a row) followed by
 `[Hkv, V, P]` values (transposed inside the page); with V = D this is the layout of the softmax attention's pages.
-HIP forms: `csrc/sigmoid_attention.hip` (any dtype and sizes, and the decode rows of every step) and, for prompt
-portions in bfloat16 with keys and values of one width 64 or 128, the matrix-core prompt kernel of
-`csrc/attention_mfma.hip` with sigmoid weights in place of its softmax."""
+HIP forms: `csrc/sigmoid_attention.hip` (any dtype and sizes) and, in bfloat16 with keys and values of one width 64
+or 128, the matrix-core prompt and decode kernels of `csrc/attention_mfma.hip` with sigmoid weights in place of
+their softmax."""
 from __future__ import annotations
 
 import ctypes
@@ -122,19 +122,21 @@ def _sigmoid_attention_hip(launch, q, pages, table, rows, token_row, positions, 
         raise ValueError(f"sigmoid_attention: q {tuple(q.shape)} {q.dtype}, pages {tuple(pages.shape)} do not fit "
                          f"{kv_heads} kv heads, values of {vdim}, page {page_size}")
     out = torch.empty((t, heads * vdim), dtype=q.dtype, device=q.device)
-    general, wide = launch
+    general, wide, narrow = launch
     common = (q.data_ptr(), out.data_ptr(), pages.data_ptr(), table.data_ptr(), table.shape[1], rows.slots.data_ptr())
     tail = (heads, kv_heads, dim, vdim, page_size, pages.shape[0], _ptr(bias), float(scale), int(window), _ptr(gate),
             _DT[q.dtype])
     on_cores = q.dtype == torch.bfloat16 and dim == vdim and dim in (64, 128) and page_size % 16 == 0 \
-        and heads // kv_heads <= 32 and rows.n_chunk > 0 and rows.max_chunk_len <= 4096 * page_size
-    if on_cores:      # prompt portions on the matrix cores, the step's decode rows (if any) in the general kernel
-        wide(*common, rows.lens.data_ptr(), rows.query_start.data_ptr(), rows.chunk_rows.data_ptr(), rows.n_chunk,
-             rows.max_chunk_query, rows.max_chunk_len, heads, kv_heads, dim, page_size, float(scale), int(window),
-             _ptr(bias), _ptr(gate))
+        and heads // kv_heads <= 32 and rows.max_chunk_len <= 4096 * page_size
+    if on_cores:      # on the matrix cores: the step's prompt portions in one launch, its decode rows in another
+        if rows.n_chunk:
+            wide(*common, rows.lens.data_ptr(), rows.query_start.data_ptr(), rows.chunk_rows.data_ptr(), rows.n_chunk,
+                 rows.max_chunk_query, rows.max_chunk_len, heads, kv_heads, dim, page_size, float(scale), int(window),
+                 _ptr(bias), _ptr(gate))
         if rows.n_decode:
-            general(*common, token_row.data_ptr(), positions.data_ptr(), rows.query_start.data_ptr(),
-                    rows.decode_rows.data_ptr(), rows.n_decode, *tail)
+            narrow(*common, rows.lens.data_ptr(), rows.query_start.data_ptr(), rows.decode_rows.data_ptr(),
+                   rows.n_decode, rows.max_decode_len, heads, kv_heads, dim, page_size, float(scale), int(window),
+                   _ptr(bias), _ptr(gate), int(rows.in_order and rows.n_decode == t))
     else:
         general(*common, token_row.data_ptr(), positions.data_ptr(), None, None, t, *tail)
     return out
@@ -144,9 +146,11 @@ register_kernel(KernelOp("head_prepare", head_prepare_plain, "holon_head_prepare
                          [_P, _P, _I, _I, _I, _I, _I, _P, _P, _F, _P, _I, _I, _P, _P, _P, _P, _I, _I, _I],
                          _head_prepare_hip))
 register_kernel(KernelOp("sigmoid_attention", sigmoid_attention_plain,
-                         ("holon_sigmoid_attention", "holon_sigmoid_attention_prefill_bf16"),
+                         ("holon_sigmoid_attention", "holon_sigmoid_attention_prefill_bf16",
+                          "holon_sigmoid_attention_decode_bf16"),
                          ([_P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P, _F, _I, _P, _I],
-                          [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P, _P]),
+                          [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P, _P],
+                          [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P, _P, _I]),
                          _sigmoid_attention_hip))
 
 
