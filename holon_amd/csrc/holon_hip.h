@@ -197,10 +197,13 @@ int holon_delta_scan(const float* qn, const float* kn, const void* qkv, int qkv_
                      const int32_t* query_start, int rows, int heads, int kv_heads, int dim, int vdim, int state_slots,
                      int dtype, void* stream);
 // The decayed key-value memory over each row's tokens; r, k, v [T, H D]; w [T, H D] float32; u [H, D];
-// state [state_slots, H, D, D] float32.
+// state [state_slots, H, D, D] float32. piece_tokens > 0: rows are cut into pieces of that many tokens that run side by
+// side in two passes (at most max_pieces a row; piece_base [rows]: the number of each row's first piece among all;
+// workspaces sloc [pieces, H, D, D] and pw [pieces, H, D], float32).
 int holon_memory_scan(const void* r, const void* k, const void* v, const float* w, const float* u, float* state,
                       float* out, const int32_t* slots, const int32_t* starts, const int32_t* query_start, int rows,
-                      int heads, int dim, int state_slots, int dtype, void* stream);
+                      int heads, int dim, int state_slots, int dtype, int piece_tokens, int max_pieces,
+                      const int32_t* piece_base, float* sloc, float* pw, void* stream);
 // y [T, H V] = o / sqrt(mean_V(o^2) + eps) * weight * silu(gate); weight [V], or [H V] with per_head.
 int holon_gated_out(const float* o, const void* gate, const void* weight, void* y, int tokens, int heads, int vdim,
                     int per_head, float eps, int dtype, void* stream);

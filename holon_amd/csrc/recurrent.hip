@@ -4,8 +4,8 @@
 // position 0 starts from zeros whatever the slot holds.
 //
 // The two scans keep a head's matrix S [D, V] in registers through a row's tokens. Its columns never meet, so a wave
-// owns 16 of them, four lanes a column with a quarter of the key rows each; what a token needs of a whole column (a dot
-// product with the key, the read-out) is summed over a lane's rows in ascending order and then over the four lanes in a
+// owns 8 of them, eight lanes a column with an eighth of the key rows each; what a token needs of a whole column (a dot
+// product with the key, the read-out) is summed over a lane's rows in ascending order and then over the eight lanes in a
 // fixed order. Each token's key and query reach the lanes through LDS. The key size is padded to the next instantiated
 // one with zeros (a zero key writes nothing).
 #include "common.h"
@@ -98,22 +98,28 @@ __global__ void __launch_bounds__(256) delta_prepare_kernel(const T* __restrict_
   }
 }
 
-// Sum over the four adjacent lanes that share a column (a fixed order: lane ^ 1, then lane ^ 2).
-__device__ __forceinline__ float quad_sum(float v) {
-  v += __shfl_xor(v, 1, WAVE);
-  v += __shfl_xor(v, 2, WAVE);
+// Sum over the eight adjacent lanes that share a column, by data-parallel moves inside the vector unit (no trip through
+// LDS): lane ^ 1, lane ^ 2, then the mirror image inside the eight, which lies in the other four. A fixed order.
+template <int CTRL> __device__ __forceinline__ float dpp_move(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float part_sum(float v) {
+  v += dpp_move<0xB1>(v);        // quad_perm [1, 0, 3, 2]
+  v += dpp_move<0x4E>(v);        // quad_perm [2, 3, 0, 1]
+  v += dpp_move<0x141>(v);       // row_half_mirror
   return v;
 }
 
-constexpr int SCAN_COLS = 16;      // value columns a wave owns; four lanes a column, each a quarter of the key rows
+constexpr int SCAN_PARTS = 8;      // lanes a value column is spread over, each with an eighth of the key rows
+constexpr int SCAN_COLS = WAVE / SCAN_PARTS;      // value columns a wave owns
 
 // Tokens a wave stages at a time: their operands travel from memory to LDS as one batch of loads while the batch before
 // is worked through, so that a token's arithmetic never waits for memory (one token at a time, a step took as long as
 // a load: 0.9 us). About a thousand values per operand and batch.
 template <int KD> struct ScanChunk { static constexpr int kTokens = KD <= 64 ? 16 : KD <= 128 ? 8 : 4; };
 
-// Per (row, head): S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q. Lane 4 c + p owns rows
-// p KD/4 .. (p + 1) KD/4 - 1 of column c of S.
+// Per (row, head): S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q. Lane 8 c + p owns rows
+// p KD/8 .. (p + 1) KD/8 - 1 of column c of S.
 template <int KD, typename T>
 __global__ void __launch_bounds__(WAVE) delta_scan_kernel(const float* __restrict__ qn, const float* __restrict__ kn,
                                                           const T* __restrict__ qkv, int qkv_stride, int v_offset,
@@ -123,12 +129,12 @@ __global__ void __launch_bounds__(WAVE) delta_scan_kernel(const float* __restric
                                                           const int32_t* __restrict__ starts,
                                                           const int32_t* __restrict__ query_start, int heads,
                                                           int kv_heads, int dim, int vdim) {
-  constexpr int KQ = KD / 4, TC = ScanChunk<KD>::kTokens, N = TC * KD, PER = (N + WAVE - 1) / WAVE;
+  constexpr int KQ = KD / SCAN_PARTS, TC = ScanChunk<KD>::kTokens, N = TC * KD, PER = (N + WAVE - 1) / WAVE;
   constexpr int VPER = (TC * SCAN_COLS + WAVE - 1) / WAVE;
   __shared__ __attribute__((aligned(16))) float ks[2][N], qs[2][N];
   __shared__ float vs[2][TC * SCAN_COLS], gs[2][TC], bs[2][TC];
   const int b = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-  const int part = lane % 4, col = lane / 4, j = blockIdx.z * SCAN_COLS + col;
+  const int part = lane % SCAN_PARTS, col = lane / SCAN_PARTS, j = blockIdx.z * SCAN_COLS + col;
   const int hk = h / (heads / kv_heads);
   const bool active = j < vdim;
   const int lo = query_start[b], hi = query_start[b + 1];
@@ -191,14 +197,14 @@ __global__ void __launch_bounds__(WAVE) delta_scan_kernel(const float* __restric
         S[i] *= gt;
         dot += S[i] * kt[i];
       }
-      const float u = bt * (vt - quad_sum(dot));
+      const float u = bt * (vt - part_sum(dot));
       float o = 0.f;
 #pragma unroll
       for (int i = 0; i < KQ; ++i) {
         S[i] += kt[i] * u;
         o += S[i] * qt[i];
       }
-      o = quad_sum(o);
+      o = part_sum(o);
       if (active && part == 0) out[((int64_t)(t0 + tt) * heads + h) * vdim + j] = o;
     }
     if (t0 + TC < hi) put(buf ^ 1);
@@ -213,6 +219,18 @@ __global__ void __launch_bounds__(WAVE) delta_scan_kernel(const float* __restric
   }
 }
 
+// A long row's tokens in pieces that run side by side (the memory's recurrence is linear in S and its decays do not
+// depend on S): every piece but a row's last first runs from S = 0 and leaves what it adds (`sloc`) and the product of
+// its decays per key row (`pw`); a small kernel then walks a row's pieces in order, S <- diag(pw) S + sloc, leaving
+// each piece's true starting state in place of `sloc`; then every piece runs again from there and writes its outputs.
+struct ScanPieces {
+  int tokens;                  // tokens a piece (0: rows are not cut)
+  int mode;                    // 1: from zero, leave sloc and pw; 2: from the true start, write outputs
+  const int32_t* base;         // [rows]: the number of row b's first piece among all pieces of the step
+  float* sloc;                 // [pieces, H, D, D]
+  float* pw;                   // [pieces, H, D]
+};
+
 // Per (row, head): o = (S + diag(u) k v^T)^T r; S <- diag(w) S + k v^T. The same split of S [D, D] over lanes.
 template <int KD, typename T>
 __global__ void __launch_bounds__(WAVE) memory_scan_kernel(const T* __restrict__ r, const T* __restrict__ k,
@@ -220,22 +238,40 @@ __global__ void __launch_bounds__(WAVE) memory_scan_kernel(const T* __restrict__
                                                            const float* __restrict__ u, float* __restrict__ state,
                                                            float* __restrict__ out, const int32_t* __restrict__ slots,
                                                            const int32_t* __restrict__ starts,
-                                                           const int32_t* __restrict__ query_start, int heads, int dim) {
-  constexpr int KQ = KD / 4, TC = ScanChunk<KD>::kTokens, N = TC * KD, PER = (N + WAVE - 1) / WAVE;
+                                                           const int32_t* __restrict__ query_start, int heads, int dim,
+                                                           ScanPieces pc) {
+  constexpr int KQ = KD / SCAN_PARTS, TC = ScanChunk<KD>::kTokens, N = TC * KD, PER = (N + WAVE - 1) / WAVE;
   constexpr int VPER = (TC * SCAN_COLS + WAVE - 1) / WAVE;
   __shared__ __attribute__((aligned(16))) float rs[2][N], ks[2][N], ws[2][N], us[KD];
   __shared__ float vs[2][TC * SCAN_COLS];
   const int b = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-  const int part = lane % 4, col = lane / 4, j = blockIdx.z * SCAN_COLS + col;
+  const int col_blocks = (dim + SCAN_COLS - 1) / SCAN_COLS;
+  const int piece = blockIdx.z / col_blocks, col_block = blockIdx.z % col_blocks;
+  const int part = lane % SCAN_PARTS, col = lane / SCAN_PARTS, j = col_block * SCAN_COLS + col;
   const bool active = j < dim;
-  const int lo = query_start[b], hi = query_start[b + 1];
+  int lo = query_start[b], hi = query_start[b + 1];
+  bool from_slot = true, to_slot = true;
+  int64_t piece_no = 0;
+  if (pc.tokens > 0) {                                   // (everything here is the same in all of the block's lanes)
+    const int pieces = (hi - lo + pc.tokens - 1) / pc.tokens;
+    if (piece >= pieces || (pc.mode == 1 && piece == pieces - 1)) return;
+    lo += piece * pc.tokens;
+    hi = min(hi, lo + pc.tokens);
+    from_slot = piece == 0;
+    to_slot = pc.mode == 2 && piece == pieces - 1;
+    piece_no = pc.base[b] + piece;
+  }
   float* held = state + ((int64_t)slots[b] * heads + h) * dim * dim;
   const bool carried = starts[b] > 0;
-  float S[KQ];
+  float S[KQ], pw[KQ];
 #pragma unroll
   for (int i = 0; i < KQ; ++i) {
     const int row = part * KQ + i;
-    S[i] = (carried && active && row < dim) ? held[(int64_t)row * dim + j] : 0.f;
+    const bool in = active && row < dim;
+    pw[i] = 1.f;
+    if (pc.tokens > 0 && pc.mode == 1) S[i] = 0.f;
+    else if (from_slot) S[i] = (carried && in) ? held[(int64_t)row * dim + j] : 0.f;
+    else S[i] = in ? pc.sloc[((piece_no - 1) * heads + h) * dim * dim + (int64_t)row * dim + j] : 0.f;
   }
   for (int i = lane; i < KD; i += WAVE) us[i] = i < dim ? u[h * dim + i] : 0.f;
   const int64_t width = (int64_t)heads * dim;
@@ -252,7 +288,7 @@ __global__ void __launch_bounds__(WAVE) memory_scan_kernel(const T* __restrict__
     }
 #pragma unroll
     for (int e = 0; e < VPER; ++e) {
-      const int idx = lane + e * WAVE, tt = idx / SCAN_COLS, jj = blockIdx.z * SCAN_COLS + idx % SCAN_COLS;
+      const int idx = lane + e * WAVE, tt = idx / SCAN_COLS, jj = col_block * SCAN_COLS + idx % SCAN_COLS;
       const bool ok = idx < TC * SCAN_COLS && t0 + tt < hi && jj < dim;
       nv[e] = ok ? Elem<T>::load(v[(int64_t)(t0 + tt) * width + h * dim + jj]) : 0.f;
     }
@@ -274,6 +310,7 @@ __global__ void __launch_bounds__(WAVE) memory_scan_kernel(const T* __restrict__
     put(0);
   }
   __syncthreads();
+  const bool local = pc.tokens > 0 && pc.mode == 1;
   for (int t0 = lo, buf = 0; t0 < hi; t0 += TC, buf ^= 1) {
     if (t0 + TC < hi) ask(t0 + TC);
     const int nt = min(TC, hi - t0);
@@ -283,6 +320,14 @@ __global__ void __launch_bounds__(WAVE) memory_scan_kernel(const T* __restrict__
       const float* kt = &ks[buf][tt * KD + part * KQ];
       const float* wt = &ws[buf][tt * KD + part * KQ];
       const float* ut = &us[part * KQ];
+      if (local) {                       // what the piece adds to S, and its decays' product; no output yet
+#pragma unroll
+        for (int i = 0; i < KQ; ++i) {
+          S[i] = wt[i] * S[i] + kt[i] * vt;
+          pw[i] *= wt[i];
+        }
+        continue;
+      }
       float o = 0.f;
 #pragma unroll
       for (int i = 0; i < KQ; ++i) {
@@ -290,17 +335,43 @@ __global__ void __launch_bounds__(WAVE) memory_scan_kernel(const T* __restrict__
         o += rt[i] * (S[i] + ut[i] * kv);
         S[i] = wt[i] * S[i] + kv;
       }
-      o = quad_sum(o);
+      o = part_sum(o);
       if (active && part == 0) out[(int64_t)(t0 + tt) * width + h * dim + j] = o;
     }
     if (t0 + TC < hi) put(buf ^ 1);
     __syncthreads();
   }
-  if (active) {
 #pragma unroll
-    for (int i = 0; i < KQ; ++i) {
-      const int row = part * KQ + i;
-      if (row < dim) held[(int64_t)row * dim + j] = S[i];
+  for (int i = 0; i < KQ; ++i) {
+    const int row = part * KQ + i;
+    if (!active || row >= dim) continue;
+    if (local) {
+      pc.sloc[(piece_no * heads + h) * dim * dim + (int64_t)row * dim + j] = S[i];
+      if (j == 0) pc.pw[(piece_no * heads + h) * dim + row] = pw[i];
+    } else if (to_slot) {
+      held[(int64_t)row * dim + j] = S[i];
+    }
+  }
+}
+
+// Between the two passes: a row's pieces in order. sloc[p] becomes the state piece p + 1 starts from.
+__global__ void __launch_bounds__(256) memory_pieces_kernel(const float* __restrict__ state,
+                                                            const int32_t* __restrict__ slots,
+                                                            const int32_t* __restrict__ starts,
+                                                            const int32_t* __restrict__ query_start, int heads, int dim,
+                                                            ScanPieces pc) {
+  const int b = blockIdx.x, h = blockIdx.y;
+  const int pieces = (query_start[b + 1] - query_start[b] + pc.tokens - 1) / pc.tokens;
+  const float* held = state + ((int64_t)slots[b] * heads + h) * dim * dim;
+  const bool carried = starts[b] > 0;
+  for (int e = threadIdx.x; e < dim * dim; e += 256) {
+    const int row = e / dim;
+    float s = carried ? held[e] : 0.f;
+    for (int p = 0; p + 1 < pieces; ++p) {
+      const int64_t at = (int64_t)pc.base[b] + p;
+      float* add = pc.sloc + (at * heads + h) * dim * dim + e;
+      s = pc.pw[(at * heads + h) * dim + row] * s + *add;
+      *add = s;
     }
   }
 }
@@ -455,7 +526,7 @@ extern "C" int holon_delta_scan(const float* qn, const float* kn, const void* qk
   HOLON_CHECK(rows <= 0x7fffffff / 2 && heads <= 65535 && state_slots > 0 && v_offset >= 0 &&
               v_offset + heads * vdim <= qkv_stride, "delta_scan: launch or row layout out of range");
   if (rows == 0) return 0;
-  const dim3 grid(rows, heads, (vdim + SCAN_COLS - 1) / SCAN_COLS);     // a wave for every 16 value columns
+  const dim3 grid(rows, heads, (vdim + SCAN_COLS - 1) / SCAN_COLS);     // a wave for every 8 value columns
   hipStream_t s = (hipStream_t)stream;
   BY_DTYPE(dtype, BY_KEY_SIZE(dim, (launch_delta<T, KD>(grid, s, qn, kn, qkv, qkv_stride, v_offset, beta, g,
                                                          state, out, slots, starts, query_start, heads, kv_heads, dim,
@@ -467,22 +538,42 @@ extern "C" int holon_delta_scan(const float* qn, const float* kn, const void* qk
 template <typename T, int KD>
 static void launch_memory(dim3 grid, hipStream_t s, const void* r, const void* k, const void* v,
                           const float* w, const float* u, float* state, float* out, const int32_t* slots,
-                          const int32_t* starts, const int32_t* qs, int heads, int dim) {
+                          const int32_t* starts, const int32_t* qs, int heads, int dim, ScanPieces pc) {
   memory_scan_kernel<KD, T><<<grid, WAVE, 0, s>>>((const T*)r, (const T*)k, (const T*)v, w, u, state, out, slots,
-                                                     starts, qs, heads, dim);
+                                                     starts, qs, heads, dim, pc);
 }
 
 extern "C" int holon_memory_scan(const void* r, const void* k, const void* v, const float* w, const float* u,
                                  float* state, float* out, const int32_t* slots, const int32_t* starts,
                                  const int32_t* query_start, int rows, int heads, int dim, int state_slots, int dtype,
+                                 int piece_tokens, int max_pieces, const int32_t* piece_base, float* sloc, float* pw,
                                  void* stream) {
   HOLON_CHECK(rows >= 0 && heads > 0 && heads <= 65535 && dim > 0 && dim <= 256 && state_slots > 0,
               "memory_scan: %d heads of %d (at most 256)", heads, dim);
+  HOLON_CHECK(piece_tokens == 0 || (piece_tokens > 0 && max_pieces > 0 && piece_base && sloc && pw),
+              "memory_scan: rows in pieces of %d tokens need the pieces' table and workspace", piece_tokens);
   if (rows == 0) return 0;
-  const dim3 grid(rows, heads, (dim + SCAN_COLS - 1) / SCAN_COLS);
+  const int col_blocks = (dim + SCAN_COLS - 1) / SCAN_COLS;
   hipStream_t s = (hipStream_t)stream;
+  ScanPieces pc{piece_tokens, 0, piece_base, sloc, pw};
+  if (piece_tokens == 0) {
+    const dim3 grid(rows, heads, col_blocks);
+    BY_DTYPE(dtype, BY_KEY_SIZE(dim, (launch_memory<T, KD>(grid, s, r, k, v, w, u, state, out, slots, starts,
+                                                            query_start, heads, dim, pc))));
+    HOLON_LAUNCH_OK();
+    return 0;
+  }
+  HOLON_CHECK((int64_t)col_blocks * max_pieces <= 65535, "memory_scan: %d pieces a row exceed one launch", max_pieces);
+  const dim3 grid(rows, heads, col_blocks * max_pieces);
+  pc.mode = 1;
   BY_DTYPE(dtype, BY_KEY_SIZE(dim, (launch_memory<T, KD>(grid, s, r, k, v, w, u, state, out, slots, starts,
-                                                          query_start, heads, dim))));
+                                                          query_start, heads, dim, pc))));
+  HOLON_LAUNCH_OK();
+  memory_pieces_kernel<<<dim3(rows, heads), 256, 0, s>>>(state, slots, starts, query_start, heads, dim, pc);
+  HOLON_LAUNCH_OK();
+  pc.mode = 2;
+  BY_DTYPE(dtype, BY_KEY_SIZE(dim, (launch_memory<T, KD>(grid, s, r, k, v, w, u, state, out, slots, starts,
+                                                          query_start, heads, dim, pc))));
   HOLON_LAUNCH_OK();
   return 0;
 }

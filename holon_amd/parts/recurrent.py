@@ -169,10 +169,11 @@ def _decay_lora_hip(launch, a, w2t, w0):
     return y
 
 
-def memory_scan_plain(r, k, v, w, u, state, slots, starts, query_start, n_rows, heads):
+def memory_scan_plain(r, k, v, w, u, state, slots, starts, query_start, n_rows, heads, pieces=None):
     """Per row and head along the row's tokens: o = (S + diag(u) k v^T)^T r, then S <- diag(w) S + k v^T.
     r, k, v [T, H D]; w [T, H D] float32 (decay per key channel); u [H, D] float32; state [slots, H, D, D] float32.
-    -> o [T, H, D] float32."""
+    -> o [T, H, D] float32. `pieces` (what `scan_pieces` answers, or None) lets a kernel run long rows in pieces side
+    by side; the result is the same but for the order of the sums."""
     t = r.shape[0]
     dim = r.shape[1] // heads
     rf, kf, vf = (x.float().view(t, heads, dim) for x in (r, k, v))
@@ -189,7 +190,21 @@ def memory_scan_plain(r, k, v, w, u, state, slots, starts, query_start, n_rows, 
     return out
 
 
-def _memory_scan_hip(launch, r, k, v, w, u, state, slots, starts, query_start, n_rows, heads):
+def scan_pieces(step, tokens: int = 128, least: int = 256):
+    """For a step with a row of `least` tokens or more (never a step replayed from a graph: those rows have one token):
+    (tokens a piece, the most pieces a row has, the number of each row's first piece among all [rows] int32 on the
+    device, pieces in all), made once a step from the host's row lengths; else None."""
+    if step.rows.max_chunk_query < least:
+        return None
+    cached = getattr(step, "_scan_pieces", None)
+    if cached is None or cached[0] != tokens:
+        n = -(-step.h_counts // tokens)
+        base = torch.from_numpy((n.cumsum() - n).astype("int32")).to(step.slots.device, non_blocking=True)
+        cached = step._scan_pieces = (tokens, int(n.max()), base, int(n.sum()))
+    return cached
+
+
+def _memory_scan_hip(launch, r, k, v, w, u, state, slots, starts, query_start, n_rows, heads, pieces=None):
     t = r.shape[0]
     dim = r.shape[1] // heads
     _need(r.is_cuda and all(x.is_contiguous() and x.dtype == r.dtype and x.shape == r.shape for x in (r, k, v))
@@ -199,9 +214,15 @@ def _memory_scan_hip(launch, r, k, v, w, u, state, slots, starts, query_start, n
           "memory_scan: shapes do not fit")
     _need(dim <= MAX_KEY_DIM, f"memory_scan: head size {dim} (at most {MAX_KEY_DIM})")
     out = torch.empty((t, heads, dim), dtype=torch.float32, device=r.device)
+    extra = (0, 0, None, None, None)
+    if pieces is not None:
+        tokens, most, base, total = pieces
+        sloc = torch.empty((total, heads, dim, dim), dtype=torch.float32, device=r.device)
+        pw = torch.empty((total, heads, dim), dtype=torch.float32, device=r.device)
+        extra = (tokens, most, base.data_ptr(), sloc.data_ptr(), pw.data_ptr())
     launch(r.data_ptr(), k.data_ptr(), v.data_ptr(), w.data_ptr(), u.data_ptr(), state.data_ptr(), out.data_ptr(),
            slots.data_ptr(), starts.data_ptr(), query_start.data_ptr(), n_rows, heads, dim, state.shape[0],
-           _DT[r.dtype])
+           _DT[r.dtype], *extra)
     return out
 
 
@@ -216,7 +237,8 @@ register_kernel(KernelOp("shift_mix", shift_mix_plain, "holon_shift_mix",
 register_kernel(KernelOp("decay_lora", decay_lora_plain, "holon_decay_lora", [_P, _P, _P, _P, _I, _I, _I, _I],
                          _decay_lora_hip))
 register_kernel(KernelOp("memory_scan", memory_scan_plain, "holon_memory_scan",
-                         [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I], _memory_scan_hip))
+                         [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P],
+                         _memory_scan_hip))
 
 
 # -- parts ------------------------------------------------------------------------------------------------------------
@@ -331,7 +353,8 @@ class DecayMemory(Part):
         r, kk, v, gate = (getattr(self, nm)(mixes[i]) for i, nm in enumerate(("r", "k", "v", "g")))
         lora = k.linear(mixes[4], self.w1, torch.float32)
         decay = k.decay_lora(lora, self.w2t, self.w0)
-        o = k.memory_scan(r, kk, v, decay, self.u, site.slot_state[self.prefix + "S"], *rows, step.n_rows, self.heads)
+        o = k.memory_scan(r, kk, v, decay, self.u, site.slot_state[self.prefix + "S"], *rows, step.n_rows, self.heads,
+                          scan_pieces(step))
         return self.o(k.gated_out(o, gate, self.norm, True, self.eps, self.build.dtype))
 
     __call__ = forward

@@ -217,6 +217,27 @@ def test_a_far_token_reaches_through_the_state(tmp_path, name, device):
 
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_long_rows_run_in_pieces(folders, dtype, device):
+    """Rows long enough for the memory's scan to cut them into pieces that run side by side: a prompt of 700 tokens
+    whole, then portions of 300 and 290 beside a short request and a decode row, then the rest token by token."""
+    folder = folders["right"]
+    vocab = M.ONLY_RIGHT["vocab"]
+    long_ids, short_ids = H.random_ids(700, vocab, 31), H.random_ids(41, vocab, 32)
+    rep = _replayer(folder, device, dtype, 16, cache_tokens=1600, max_model_len=704)
+    got = H.run_trace(rep, H.trace_whole({"long": long_ids}))
+    _check(folder, dtype, {"long": long_ids}, got, f"pieces, whole {dtype}")
+    trace = H.Trace()
+    trace.add([("long", 0, long_ids[:300], [0, 127, 128, 255, 256, 299]), ("short", 0, short_ids[:40], [39])])
+    trace.add([("long", 300, long_ids[300:590], [0, 100, 289]), ("short", 40, short_ids[40:], [0])], end=["short"])
+    for at in range(590, 700):
+        trace.add([("long", at, [long_ids[at]], [0])], end=["long"] if at == 699 else [])
+    got = H.run_trace(rep, trace)
+    _check(folder, dtype, {"long": long_ids, "short": short_ids}, got, f"pieces, portions {dtype}")
+    rep.cache.check()
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_long_decoding(folders, dtype, device):
     """180 tokens one by one after a prompt of 5: many window lengths, many pages given back on the way."""
     folder, page = folders["X-sharp"], 8
