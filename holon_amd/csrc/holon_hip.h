@@ -192,10 +192,13 @@ int holon_delta_prepare(const void* qkv, const void* ab, const float* a_log, con
                         float* beta, float* g, int tokens, int heads, int kv_heads, int dim, int vdim, int dtype,
                         void* stream);
 // The gated delta rule over each row's tokens; v = qkv[t, v_offset + h V + j]; state [state_slots, H, D, V] float32.
+// piece_tokens > 0: rows in pieces that run side by side, as for holon_memory_scan; workspaces ab [pieces, H, D, V + D]
+// and sin [pieces, H, D, V], float32.
 int holon_delta_scan(const float* qn, const float* kn, const void* qkv, int qkv_stride, int v_offset, const float* beta,
                      const float* g, float* state, float* out, const int32_t* slots, const int32_t* starts,
                      const int32_t* query_start, int rows, int heads, int kv_heads, int dim, int vdim, int state_slots,
-                     int dtype, void* stream);
+                     int dtype, int piece_tokens, int max_pieces, const int32_t* piece_base, float* ab, float* sin,
+                     void* stream);
 // The decayed key-value memory over each row's tokens; r, k, v [T, H D]; w [T, H D] float32; u [H, D];
 // state [state_slots, H, D, D] float32. piece_tokens > 0: rows are cut into pieces of that many tokens that run side by
 // side in two passes (at most max_pieces a row; piece_base [rows]: the number of each row's first piece among all;

@@ -116,7 +116,25 @@ constexpr int SCAN_COLS = WAVE / SCAN_PARTS;      // value columns a wave owns
 // Tokens a wave stages at a time: their operands travel from memory to LDS as one batch of loads while the batch before
 // is worked through, so that a token's arithmetic never waits for memory (one token at a time, a step took as long as
 // a load: 0.9 us). About a thousand values per operand and batch.
-template <int KD> struct ScanChunk { static constexpr int kTokens = KD <= 64 ? 16 : KD <= 128 ? 8 : 4; };
+// ARRAYS: operands of D values a token that the scan stages (they decide the block's LDS, and with it how many waves a
+// compute unit holds: the scans wait on latencies, so more waves are more throughput).
+template <int KD, int ARRAYS> struct ScanChunk {
+  static constexpr int kTokens = ARRAYS <= 2 ? (KD <= 64 ? 16 : KD <= 128 ? 8 : 4) : (KD <= 64 ? 8 : KD <= 128 ? 4 : 2);
+};
+
+// A long row's tokens in pieces that run side by side, for the delta rule. A token's step is linear in S,
+// S <- g (I - beta k k^T) S + beta k v^T, with a matrix in front that does not depend on S. Every piece but a row's last
+// first runs on D + V columns: V from zero with the true values (what the piece adds, B) and D from the identity with
+// values of zero (the product of its matrices, A); `ab` [pieces, H, D, V + D] takes both. A small kernel walks a row's
+// pieces in order, S <- A S + B, leaving each piece's true starting state in `sin` [pieces, H, D, V]; then every piece
+// runs again from there and writes its outputs.
+struct DeltaPieces {
+  int tokens;                  // tokens a piece (0: rows are not cut)
+  int mode;                    // 1: B and A of every piece but the last; 2: from the true start, outputs
+  const int32_t* base;         // [rows]: the number of row b's first piece among all pieces of the step
+  float* ab;
+  float* sin;
+};
 
 // Per (row, head): S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q. Lane 8 c + p owns rows
 // p KD/8 .. (p + 1) KD/8 - 1 of column c of S.
@@ -128,23 +146,41 @@ __global__ void __launch_bounds__(WAVE) delta_scan_kernel(const float* __restric
                                                           const int32_t* __restrict__ slots,
                                                           const int32_t* __restrict__ starts,
                                                           const int32_t* __restrict__ query_start, int heads,
-                                                          int kv_heads, int dim, int vdim) {
-  constexpr int KQ = KD / SCAN_PARTS, TC = ScanChunk<KD>::kTokens, N = TC * KD, PER = (N + WAVE - 1) / WAVE;
+                                                          int kv_heads, int dim, int vdim, DeltaPieces pc) {
+  constexpr int KQ = KD / SCAN_PARTS, TC = ScanChunk<KD, 2>::kTokens, N = TC * KD, PER = (N + WAVE - 1) / WAVE;
   constexpr int VPER = (TC * SCAN_COLS + WAVE - 1) / WAVE;
   __shared__ __attribute__((aligned(16))) float ks[2][N], qs[2][N];
   __shared__ float vs[2][TC * SCAN_COLS], gs[2][TC], bs[2][TC];
   const int b = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-  const int part = lane % SCAN_PARTS, col = lane / SCAN_PARTS, j = blockIdx.z * SCAN_COLS + col;
+  const bool local = pc.tokens > 0 && pc.mode == 1;
+  const int columns = local ? vdim + dim : vdim;          // the first pass also carries the identity's D columns
+  const int col_blocks = (columns + SCAN_COLS - 1) / SCAN_COLS;
+  const int piece = blockIdx.z / col_blocks, col_block = blockIdx.z % col_blocks;
+  const int part = lane % SCAN_PARTS, col = lane / SCAN_PARTS, j = col_block * SCAN_COLS + col;
   const int hk = h / (heads / kv_heads);
-  const bool active = j < vdim;
-  const int lo = query_start[b], hi = query_start[b + 1];
+  const bool active = j < columns;
+  int lo = query_start[b], hi = query_start[b + 1];
+  bool from_slot = true, to_slot = true;
+  int64_t piece_no = 0;
+  if (pc.tokens > 0) {                                   // (everything here is the same in all of the block's lanes)
+    const int pieces = (hi - lo + pc.tokens - 1) / pc.tokens;
+    if (piece >= pieces || (local && piece == pieces - 1)) return;
+    lo += piece * pc.tokens;
+    hi = min(hi, lo + pc.tokens);
+    from_slot = piece == 0;
+    to_slot = pc.mode == 2 && piece == pieces - 1;
+    piece_no = pc.base[b] + piece;
+  }
   float* held = state + ((int64_t)slots[b] * heads + h) * dim * vdim;
   const bool carried = starts[b] > 0;
   float S[KQ];
 #pragma unroll
   for (int i = 0; i < KQ; ++i) {
     const int row = part * KQ + i;
-    S[i] = (carried && active && row < dim) ? held[(int64_t)row * vdim + j] : 0.f;
+    const bool in = active && row < dim;
+    if (local) S[i] = (in && j >= vdim && row == j - vdim) ? 1.f : 0.f;
+    else if (from_slot) S[i] = (carried && in) ? held[(int64_t)row * vdim + j] : 0.f;
+    else S[i] = in ? pc.sin[((piece_no - 1) * heads + h) * dim * vdim + (int64_t)row * vdim + j] : 0.f;
   }
   float nk[PER], nq[PER], nv[VPER], ng = 1.f, nb = 0.f;
   auto ask = [&](int t0) {
@@ -158,8 +194,8 @@ __global__ void __launch_bounds__(WAVE) delta_scan_kernel(const float* __restric
     }
 #pragma unroll
     for (int e = 0; e < VPER; ++e) {
-      const int idx = lane + e * WAVE, tt = idx / SCAN_COLS, jj = blockIdx.z * SCAN_COLS + idx % SCAN_COLS;
-      const bool ok = idx < TC * SCAN_COLS && t0 + tt < hi && jj < vdim;
+      const int idx = lane + e * WAVE, tt = idx / SCAN_COLS, jj = col_block * SCAN_COLS + idx % SCAN_COLS;
+      const bool ok = idx < TC * SCAN_COLS && t0 + tt < hi && jj < vdim;      // (the identity's columns take v = 0)
       nv[e] = ok ? Elem<T>::load(qkv[(int64_t)(t0 + tt) * qkv_stride + v_offset + h * vdim + jj]) : 0.f;
     }
     const bool ok = lane < TC && t0 + lane < hi;
@@ -198,6 +234,11 @@ __global__ void __launch_bounds__(WAVE) delta_scan_kernel(const float* __restric
         dot += S[i] * kt[i];
       }
       const float u = bt * (vt - part_sum(dot));
+      if (local) {
+#pragma unroll
+        for (int i = 0; i < KQ; ++i) S[i] += kt[i] * u;
+        continue;
+      }
       float o = 0.f;
 #pragma unroll
       for (int i = 0; i < KQ; ++i) {
@@ -210,11 +251,70 @@ __global__ void __launch_bounds__(WAVE) delta_scan_kernel(const float* __restric
     if (t0 + TC < hi) put(buf ^ 1);
     __syncthreads();
   }
-  if (active) {
 #pragma unroll
-    for (int i = 0; i < KQ; ++i) {
-      const int row = part * KQ + i;
-      if (row < dim) held[(int64_t)row * vdim + j] = S[i];
+  for (int i = 0; i < KQ; ++i) {
+    const int row = part * KQ + i;
+    if (!active || row >= dim) continue;
+    if (local) pc.ab[((piece_no * heads + h) * dim + row) * (int64_t)(vdim + dim) + j] = S[i];
+    else if (to_slot) held[(int64_t)row * vdim + j] = S[i];
+  }
+}
+
+// Between the two passes: a row's pieces in order, S <- A S + B, sixteen columns of S a block (columns never meet).
+// A comes through LDS in slabs of 32 columns, S's sixteen columns stay there. sin[p] becomes the state piece p + 1
+// starts from.
+__global__ void __launch_bounds__(256) delta_pieces_kernel(const float* __restrict__ state,
+                                                           const int32_t* __restrict__ slots,
+                                                           const int32_t* __restrict__ starts,
+                                                           const int32_t* __restrict__ query_start, int heads, int dim,
+                                                           int vdim, DeltaPieces pc) {
+  constexpr int SLAB = 32, MAXD = 256, PER = MAXD * 16 / 256;
+  __shared__ float sc[MAXD * 16];
+  __shared__ float as[MAXD][SLAB + 1];
+  const int b = blockIdx.x, h = blockIdx.y, j0 = blockIdx.z * 16;
+  const int pieces = (query_start[b + 1] - query_start[b] + pc.tokens - 1) / pc.tokens;
+  const float* held = state + ((int64_t)slots[b] * heads + h) * dim * vdim;
+  const bool carried = starts[b] > 0;
+  for (int e = threadIdx.x; e < dim * 16; e += 256) {
+    const int m = e / 16, j = j0 + e % 16;
+    sc[e] = carried && j < vdim ? held[(int64_t)m * vdim + j] : 0.f;
+  }
+  for (int p = 0; p + 1 < pieces; ++p) {
+    const int64_t at = ((int64_t)pc.base[b] + p) * heads + h;
+    const float* ab = pc.ab + at * dim * (vdim + dim);
+    float* next = pc.sin + at * dim * vdim;
+    float acc[PER];
+#pragma unroll
+    for (int k = 0; k < PER; ++k) {                      // element e = threadIdx.x + 256 k: row e / 16, column e % 16
+      const int e = threadIdx.x + 256 * k, i = e / 16, j = j0 + e % 16;
+      acc[k] = e < dim * 16 && j < vdim ? ab[(int64_t)i * (vdim + dim) + j] : 0.f;
+    }
+    for (int m0 = 0; m0 < dim; m0 += SLAB) {
+      __syncthreads();                                   // the slab before, and S, are settled
+      for (int e = threadIdx.x; e < dim * SLAB; e += 256) {
+        const int i = e / SLAB, m = e % SLAB;
+        as[i][m] = m0 + m < dim ? ab[(int64_t)i * (vdim + dim) + vdim + m0 + m] : 0.f;
+      }
+      __syncthreads();
+      const int span = min(SLAB, dim - m0);
+#pragma unroll
+      for (int k = 0; k < PER; ++k) {
+        const int e = threadIdx.x + 256 * k, i = e / 16, c = e % 16;
+        if (e < dim * 16) {
+          float a = acc[k];
+          for (int m = 0; m < span; ++m) a += as[i][m] * sc[(m0 + m) * 16 + c];
+          acc[k] = a;
+        }
+      }
+    }
+    __syncthreads();                                     // every thread has read the old S
+#pragma unroll
+    for (int k = 0; k < PER; ++k) {
+      const int e = threadIdx.x + 256 * k, i = e / 16, j = j0 + e % 16;
+      if (e < dim * 16) {
+        sc[e] = acc[k];
+        if (j < vdim) next[(int64_t)i * vdim + j] = acc[k];
+      }
     }
   }
 }
@@ -240,7 +340,7 @@ __global__ void __launch_bounds__(WAVE) memory_scan_kernel(const T* __restrict__
                                                            const int32_t* __restrict__ starts,
                                                            const int32_t* __restrict__ query_start, int heads, int dim,
                                                            ScanPieces pc) {
-  constexpr int KQ = KD / SCAN_PARTS, TC = ScanChunk<KD>::kTokens, N = TC * KD, PER = (N + WAVE - 1) / WAVE;
+  constexpr int KQ = KD / SCAN_PARTS, TC = ScanChunk<KD, 3>::kTokens, N = TC * KD, PER = (N + WAVE - 1) / WAVE;
   constexpr int VPER = (TC * SCAN_COLS + WAVE - 1) / WAVE;
   __shared__ __attribute__((aligned(16))) float rs[2][N], ks[2][N], ws[2][N], us[KD];
   __shared__ float vs[2][TC * SCAN_COLS];
@@ -499,9 +599,9 @@ template <typename T, int KD>
 static void launch_delta(dim3 grid, hipStream_t s, const float* qn, const float* kn, const void* qkv,
                          int stride, int voff, const float* beta, const float* g, float* state, float* out,
                          const int32_t* slots, const int32_t* starts, const int32_t* qs, int heads, int kv_heads, int dim,
-                         int vdim) {
+                         int vdim, DeltaPieces pc) {
   delta_scan_kernel<KD, T><<<grid, WAVE, 0, s>>>(qn, kn, (const T*)qkv, stride, voff, beta, g, state, out, slots,
-                                                    starts, qs, heads, kv_heads, dim, vdim);
+                                                    starts, qs, heads, kv_heads, dim, vdim, pc);
 }
 
 #define BY_KEY_SIZE(dim, CALL)                                  \
@@ -519,18 +619,41 @@ static void launch_delta(dim3 grid, hipStream_t s, const float* qn, const float*
 extern "C" int holon_delta_scan(const float* qn, const float* kn, const void* qkv, int qkv_stride, int v_offset,
                                 const float* beta, const float* g, float* state, float* out, const int32_t* slots,
                                 const int32_t* starts, const int32_t* query_start, int rows, int heads, int kv_heads,
-                                int dim, int vdim, int state_slots, int dtype, void* stream) {
+                                int dim, int vdim, int state_slots, int dtype, int piece_tokens, int max_pieces,
+                                const int32_t* piece_base, float* ab, float* sin, void* stream) {
   HOLON_CHECK(rows >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "delta_scan: %d/%d heads", heads, kv_heads);
   HOLON_CHECK(dim > 0 && dim <= 256 && vdim > 0 && vdim <= 1024, "delta_scan: key size %d (at most 256), value size %d "
               "(at most 1024)", dim, vdim);
   HOLON_CHECK(rows <= 0x7fffffff / 2 && heads <= 65535 && state_slots > 0 && v_offset >= 0 &&
               v_offset + heads * vdim <= qkv_stride, "delta_scan: launch or row layout out of range");
+  HOLON_CHECK(piece_tokens == 0 || (piece_tokens > 0 && max_pieces > 0 && piece_base && ab && sin),
+              "delta_scan: rows in pieces of %d tokens need the pieces' table and workspace", piece_tokens);
   if (rows == 0) return 0;
-  const dim3 grid(rows, heads, (vdim + SCAN_COLS - 1) / SCAN_COLS);     // a wave for every 8 value columns
   hipStream_t s = (hipStream_t)stream;
-  BY_DTYPE(dtype, BY_KEY_SIZE(dim, (launch_delta<T, KD>(grid, s, qn, kn, qkv, qkv_stride, v_offset, beta, g,
-                                                         state, out, slots, starts, query_start, heads, kv_heads, dim,
-                                                         vdim))));
+  DeltaPieces pc{piece_tokens, 0, piece_base, ab, sin};
+  const int col_blocks = (vdim + SCAN_COLS - 1) / SCAN_COLS;     // a wave for every 8 value columns
+  if (piece_tokens == 0) {
+    const dim3 grid(rows, heads, col_blocks);
+    BY_DTYPE(dtype, BY_KEY_SIZE(dim, (launch_delta<T, KD>(grid, s, qn, kn, qkv, qkv_stride, v_offset, beta, g, state,
+                                                           out, slots, starts, query_start, heads, kv_heads, dim, vdim,
+                                                           pc))));
+    HOLON_LAUNCH_OK();
+    return 0;
+  }
+  const int col_blocks_first = (vdim + dim + SCAN_COLS - 1) / SCAN_COLS;
+  HOLON_CHECK((int64_t)col_blocks_first * max_pieces <= 65535, "delta_scan: %d pieces a row exceed one launch", max_pieces);
+  pc.mode = 1;
+  BY_DTYPE(dtype, BY_KEY_SIZE(dim, (launch_delta<T, KD>(dim3(rows, heads, col_blocks_first * max_pieces), s, qn, kn, qkv,
+                                                         qkv_stride, v_offset, beta, g, state, out, slots, starts,
+                                                         query_start, heads, kv_heads, dim, vdim, pc))));
+  HOLON_LAUNCH_OK();
+  delta_pieces_kernel<<<dim3(rows, heads, (vdim + 15) / 16), 256, 0, s>>>(state, slots, starts, query_start, heads, dim,
+                                                                          vdim, pc);
+  HOLON_LAUNCH_OK();
+  pc.mode = 2;
+  BY_DTYPE(dtype, BY_KEY_SIZE(dim, (launch_delta<T, KD>(dim3(rows, heads, col_blocks * max_pieces), s, qn, kn, qkv,
+                                                         qkv_stride, v_offset, beta, g, state, out, slots, starts,
+                                                         query_start, heads, kv_heads, dim, vdim, pc))));
   HOLON_LAUNCH_OK();
   return 0;
 }

@@ -65,10 +65,10 @@ def _delta_prepare_hip(launch, qkv, ab, a_log, dt_bias, heads, kv_heads, dim, vd
     return qn, kn, beta, g
 
 
-def delta_scan_plain(qn, kn, qkv, beta, g, state, slots, starts, query_start, n_rows, heads, vdim):
+def delta_scan_plain(qn, kn, qkv, beta, g, state, slots, starts, query_start, n_rows, heads, vdim, pieces=None):
     """Per row and head, along the row's tokens: S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q.
     qn, kn [T, G, D] float32; v is the last H V columns of qkv; state [slots, H, D, V] float32, read unless the row
-    starts at position 0 and written back. -> o [T, H, V] float32."""
+    starts at position 0 and written back. -> o [T, H, V] float32. `pieces` as for `memory_scan`."""
     t, kv_heads, dim = qn.shape
     v = qkv[:, qkv.shape[1] - heads * vdim:].float().view(t, heads, vdim)
     out = torch.empty((t, heads, vdim), dtype=torch.float32, device=qn.device)
@@ -87,7 +87,7 @@ def delta_scan_plain(qn, kn, qkv, beta, g, state, slots, starts, query_start, n_
     return out
 
 
-def _delta_scan_hip(launch, qn, kn, qkv, beta, g, state, slots, starts, query_start, n_rows, heads, vdim):
+def _delta_scan_hip(launch, qn, kn, qkv, beta, g, state, slots, starts, query_start, n_rows, heads, vdim, pieces=None):
     t, kv_heads, dim = qn.shape
     _need(qn.is_cuda and qn.dtype == torch.float32 and kn.dtype == torch.float32 and qn.is_contiguous()
           and kn.is_contiguous() and qkv.is_contiguous() and qkv.dtype in _DT and beta.is_contiguous()
@@ -97,9 +97,15 @@ def _delta_scan_hip(launch, qn, kn, qkv, beta, g, state, slots, starts, query_st
     _need(dim <= MAX_KEY_DIM and vdim <= 1024, f"delta_scan: key size {dim} (at most {MAX_KEY_DIM}), value size {vdim} "
           "(at most 1024)")
     out = torch.empty((t, heads, vdim), dtype=torch.float32, device=qn.device)
+    extra = (0, 0, None, None, None)
+    if pieces is not None:
+        tokens, most, base, total = pieces
+        ab = torch.empty((total, heads, dim, vdim + dim), dtype=torch.float32, device=qn.device)
+        sin = torch.empty((total, heads, dim, vdim), dtype=torch.float32, device=qn.device)
+        extra = (tokens, most, base.data_ptr(), ab.data_ptr(), sin.data_ptr())
     launch(qn.data_ptr(), kn.data_ptr(), qkv.data_ptr(), qkv.shape[1], qkv.shape[1] - heads * vdim, beta.data_ptr(),
            g.data_ptr(), state.data_ptr(), out.data_ptr(), slots.data_ptr(), starts.data_ptr(), query_start.data_ptr(),
-           n_rows, heads, kv_heads, dim, vdim, state.shape[0], _DT[qkv.dtype])
+           n_rows, heads, kv_heads, dim, vdim, state.shape[0], _DT[qkv.dtype], *extra)
     return out
 
 
@@ -229,7 +235,8 @@ def _memory_scan_hip(launch, r, k, v, w, u, state, slots, starts, query_start, n
 register_kernel(KernelOp("delta_prepare", delta_prepare_plain, "holon_delta_prepare",
                          [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I], _delta_prepare_hip))
 register_kernel(KernelOp("delta_scan", delta_scan_plain, "holon_delta_scan",
-                         [_P, _P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I], _delta_scan_hip))
+                         [_P, _P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P],
+                         _delta_scan_hip))
 register_kernel(KernelOp("gated_out", gated_out_plain, "holon_gated_out", [_P, _P, _P, _P, _I, _I, _I, _I, _F, _I],
                          _gated_out_hip))
 register_kernel(KernelOp("shift_mix", shift_mix_plain, "holon_shift_mix",
@@ -295,7 +302,7 @@ class GatedDelta(Part):
         qn, kn, beta, g = k.delta_prepare(qkv, self.ab(x), self.A_log, self.dt_bias, self.heads, self.kv_heads,
                                           self.dim, self.vdim)
         o = k.delta_scan(qn, kn, qkv, beta, g, site.slot_state[self.prefix + "S"], step.slots, step.starts,
-                         step.query_start, step.n_rows, self.heads, self.vdim)
+                         step.query_start, step.n_rows, self.heads, self.vdim, scan_pieces(step))
         return self.o(k.gated_out(o, self.g(x), self.norm, False, self.eps, self.build.dtype))
 
     __call__ = forward

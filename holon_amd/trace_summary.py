@@ -24,7 +24,14 @@ SHORT = (("_Z18gemm_skinny_kernelILi", "gemm_skinny<"), ("_Z22gemm_skinny_glu_ke
          ("_Z23argmax_of_pieces_kernel", "argmax_of_pieces"), ("_Z16embedding_kernel", "embedding"),
          ("_Z15gemm_f32_kernel", "gemm_f32"), ("_Z13sample_kernel", "sample"),
          ("_ZN12_GLOBAL__N_116gemm_rows_kernelILi", "gemm_rows<"),
-         ("_Z19silu_mul_vec_kernel", "silu_mul_vec"), ("Cijk_Alik_Bljk_BBS_BH_Bias_HA_S_SAV_UserArgs_", "hipBLASLt "),
+         ("_Z19silu_mul_vec_kernel", "silu_mul_vec"), ("_ZN12_GLOBAL__N_118memory_scan_kernelILi", "memory_scan<"),
+         ("_ZN12_GLOBAL__N_117delta_scan_kernelILi", "delta_scan<"), ("_ZN12_GLOBAL__N_118stream_norm_kernelILi", "stream_norm<"),
+         ("_ZN12_GLOBAL__N_124sigmoid_attention_kernelI", "sigmoid_attention<"),
+         ("_ZN12_GLOBAL__N_118causal_conv_kernelI", "causal_conv<"), ("_ZN12_GLOBAL__N_123causal_conv_keep_kernelI", "causal_conv_keep<"),
+         ("_ZN12_GLOBAL__N_119head_prepare_kernelI", "head_prepare<"), ("_ZN12_GLOBAL__N_120delta_prepare_kernelI", "delta_prepare<"),
+         ("_ZN12_GLOBAL__N_116gated_out_kernelI", "gated_out<"), ("_ZN12_GLOBAL__N_116shift_mix_kernelI", "shift_mix<"),
+         ("_ZN12_GLOBAL__N_117shift_keep_kernelI", "shift_keep<"), ("_ZN12_GLOBAL__N_117decay_lora_kernelI", "decay_lora<"),
+         ("_ZN12_GLOBAL__N_120memory_pieces_kernel", "memory_pieces"), ("Cijk_Alik_Bljk_BBS_BH_Bias_HA_S_SAV_UserArgs_", "hipBLASLt "),
          ("Custom_Cijk_Alik_Bljk_BBS_BH_Bias_HA_S_SAV_NTD_SK3_UserArgs_", "hipBLASLt custom "))
 
 
@@ -45,9 +52,11 @@ def dispatches(path: str) -> list[tuple]:
     return [(n, st, en, gx // max(wx, 1), gy, gz) for n, st, en, gx, gy, gz, wx in rows]
 
 
-CLASSES = (("attention", ("attn_",)), ("matrix products", ("gemm_", "Cijk_", "Custom_Cijk_", "hipBLASLt")),
+CLASSES = (("attention", ("attn_", "sigmoid_attention")), ("matrix products", ("gemm_", "Cijk_", "Custom_Cijk_", "hipBLASLt")),
+           ("recurrent scans", ("memory_scan", "delta_scan", "memory_pieces", "delta_pieces")),
            ("elementwise", ("rmsnorm", "silu_mul", "qk_norm_rope", "v_write", "kv_write", "embedding", "sum_parts",
-                            "row_sumsq", "scatter_rows")),
+                            "row_sumsq", "scatter_rows", "stream_norm", "widen_", "pair_rows", "softcap", "causal_conv",
+                            "head_prepare", "delta_prepare", "gated_out", "shift_mix", "shift_keep", "decay_lora")),
            ("sampling", ("argmax", "sample_kernel", "store_tokens", "logprobs")))
 
 

@@ -217,11 +217,12 @@ def test_a_far_token_reaches_through_the_state(tmp_path, name, device):
 
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_long_rows_run_in_pieces(folders, dtype, device):
-    """Rows long enough for the memory's scan to cut them into pieces that run side by side: a prompt of 700 tokens
-    whole, then portions of 300 and 290 beside a short request and a decode row, then the rest token by token."""
-    folder = folders["right"]
-    vocab = M.ONLY_RIGHT["vocab"]
+@pytest.mark.parametrize("name", ["right", "delta", "X"])
+def test_long_rows_run_in_pieces(folders, name, dtype, device):
+    """Rows long enough for the scans to cut them into pieces that run side by side: a prompt of 700 tokens whole,
+    then portions of 300 and 290 beside a short request and a decode row, then the rest token by token."""
+    folder = folders[name]
+    vocab = MODELS[name][0]["vocab"]
     long_ids, short_ids = H.random_ids(700, vocab, 31), H.random_ids(41, vocab, 32)
     rep = _replayer(folder, device, dtype, 16, cache_tokens=1600, max_model_len=704)
     got = H.run_trace(rep, H.trace_whole({"long": long_ids}))
