@@ -275,10 +275,12 @@ __global__ void __launch_bounds__(256) delta_pieces_kernel(const float* __restri
   const int pieces = (query_start[b + 1] - query_start[b] + pc.tokens - 1) / pc.tokens;
   const float* held = state + ((int64_t)slots[b] * heads + h) * dim * vdim;
   const bool carried = starts[b] > 0;
-  for (int e = threadIdx.x; e < dim * 16; e += 256) {
+  for (int e = threadIdx.x; e < MAXD * 16; e += 256) {      // (rows from dim on stay zero: the slabs reach past dim)
     const int m = e / 16, j = j0 + e % 16;
-    sc[e] = carried && j < vdim ? held[(int64_t)m * vdim + j] : 0.f;
+    sc[e] = carried && m < dim && j < vdim ? held[(int64_t)m * vdim + j] : 0.f;
   }
+  for (int e = dim * SLAB + threadIdx.x; e < MAXD * SLAB; e += 256) as[e / SLAB][e % SLAB] = 0.f;   // rows no slab fills
+  const int c = threadIdx.x % 16;                            // this thread's column of the sixteen, whatever k
   for (int p = 0; p + 1 < pieces; ++p) {
     const int64_t at = ((int64_t)pc.base[b] + p) * heads + h;
     const float* ab = pc.ab + at * dim * (vdim + dim);
@@ -296,15 +298,11 @@ __global__ void __launch_bounds__(256) delta_pieces_kernel(const float* __restri
         as[i][m] = m0 + m < dim ? ab[(int64_t)i * (vdim + dim) + vdim + m0 + m] : 0.f;
       }
       __syncthreads();
-      const int span = min(SLAB, dim - m0);
 #pragma unroll
-      for (int k = 0; k < PER; ++k) {
-        const int e = threadIdx.x + 256 * k, i = e / 16, c = e % 16;
-        if (e < dim * 16) {
-          float a = acc[k];
-          for (int m = 0; m < span; ++m) a += as[i][m] * sc[(m0 + m) * 16 + c];
-          acc[k] = a;
-        }
+      for (int m = 0; m < SLAB; ++m) {                   // (A is zero past dim, and so are S's rows there)
+        const float sv = sc[(m0 + m) * 16 + c];
+#pragma unroll
+        for (int k = 0; k < PER; ++k) acc[k] += as[threadIdx.x / 16 + 16 * k][m] * sv;
       }
     }
     __syncthreads();                                     // every thread has read the old S
