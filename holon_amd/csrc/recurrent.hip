@@ -293,9 +293,16 @@ __global__ void __launch_bounds__(256) delta_pieces_kernel(const float* __restri
     }
     for (int m0 = 0; m0 < dim; m0 += SLAB) {
       __syncthreads();                                   // the slab before, and S, are settled
-      for (int e = threadIdx.x; e < dim * SLAB; e += 256) {
-        const int i = e / SLAB, m = e % SLAB;
-        as[i][m] = m0 + m < dim ? ab[(int64_t)i * (vdim + dim) + vdim + m0 + m] : 0.f;
+      float slab[MAXD * SLAB / 256];                     // all of a thread's loads under way before the first is used
+#pragma unroll
+      for (int k = 0; k < MAXD * SLAB / 256; ++k) {
+        const int e = threadIdx.x + 256 * k, i = e / SLAB, m = e % SLAB;
+        slab[k] = e < dim * SLAB && m0 + m < dim ? ab[(int64_t)i * (vdim + dim) + vdim + m0 + m] : 0.f;
+      }
+#pragma unroll
+      for (int k = 0; k < MAXD * SLAB / 256; ++k) {
+        const int e = threadIdx.x + 256 * k;
+        if (e < dim * SLAB) as[e / SLAB][e % SLAB] = slab[k];
       }
       __syncthreads();
 #pragma unroll
