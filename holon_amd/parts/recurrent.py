@@ -199,15 +199,17 @@ def memory_scan_plain(r, k, v, w, u, state, slots, starts, query_start, n_rows, 
 def scan_pieces(step, tokens: int = 128, least: int = 256):
     """For a step with a row of `least` tokens or more (never a step replayed from a graph: those rows have one token):
     (tokens a piece, the most pieces a row has, the number of each row's first piece among all [rows] int32 on the
-    device, pieces in all), made once a step from the host's row lengths; else None."""
+    device, pieces in all), made once a step and piece length from the host's row lengths; else None. (The delta
+    rule takes pieces of 256 tokens: the ordered walk between its two passes multiplies matrices, and is the shorter
+    the fewer pieces there are.)"""
     if step.rows.max_chunk_query < least:
         return None
-    cached = getattr(step, "_scan_pieces", None)
-    if cached is None or cached[0] != tokens:
+    cache = step.__dict__.setdefault("_scan_pieces", {})
+    if tokens not in cache:
         n = -(-step.h_counts // tokens)
         base = torch.from_numpy((n.cumsum() - n).astype("int32")).to(step.slots.device, non_blocking=True)
-        cached = step._scan_pieces = (tokens, int(n.max()), base, int(n.sum()))
-    return cached
+        cache[tokens] = (tokens, int(n.max()), base, int(n.sum()))
+    return cache[tokens]
 
 
 def _memory_scan_hip(launch, r, k, v, w, u, state, slots, starts, query_start, n_rows, heads, pieces=None):
@@ -302,7 +304,7 @@ class GatedDelta(Part):
         qn, kn, beta, g = k.delta_prepare(qkv, self.ab(x), self.A_log, self.dt_bias, self.heads, self.kv_heads,
                                           self.dim, self.vdim)
         o = k.delta_scan(qn, kn, qkv, beta, g, site.slot_state[self.prefix + "S"], step.slots, step.starts,
-                         step.query_start, step.n_rows, self.heads, self.vdim, scan_pieces(step))
+                         step.query_start, step.n_rows, self.heads, self.vdim, scan_pieces(step, 256, 512))
         return self.o(k.gated_out(o, self.g(x), self.norm, False, self.eps, self.build.dtype))
 
     __call__ = forward
