@@ -183,9 +183,10 @@ int holon_softcap(float* logits, int64_t n, float cap, void* stream);
 // -- recurrent mixers (recurrent.hip); rows are ranges query_start[b] .. query_start[b + 1] of the flat tokens ----------
 // y_t[c] = act(sum_j w[c, j] x_(t - taps + 1 + j)[c] (+ x_t[c])); state [state_slots, taps - 1, channels] holds each
 // request's last inputs (ignored by a row that starts at 0) and takes the row's last ones afterwards.
+// rows_in_order: every row has one token and token t is row t (a decode step): one kernel then does both.
 int holon_causal_conv(const void* x, const void* w, void* state, void* y, const int32_t* slots, const int32_t* starts,
                       const int32_t* query_start, const int32_t* token_row, int tokens, int rows, int channels, int taps,
-                      int state_slots, int add_input, int act, int dtype, void* stream);
+                      int state_slots, int add_input, int act, int dtype, int rows_in_order, void* stream);
 // From filtered q, k, v [T, 2 G D + H V] and the projections ab [T, 2 H]: unit q (times D^-0.5) and k [T, G, D],
 // beta = sigmoid(b), g = exp(-exp(a_log) softplus(a + dt_bias)) [T, H]; all outputs float32.
 int holon_delta_prepare(const void* qkv, const void* ab, const float* a_log, const float* dt_bias, float* qn, float* kn,
@@ -214,7 +215,7 @@ int holon_gated_out(const float* o, const void* gate, const void* weight, void* 
 // token, zeros for a row that starts at 0); the state then takes each row's last x.
 int holon_shift_mix(const void* x, const void* mu, void* state, void* y, const int32_t* slots, const int32_t* starts,
                     const int32_t* query_start, const int32_t* token_row, int tokens, int rows, int width, int mixes,
-                    int state_slots, int dtype, void* stream);
+                    int state_slots, int dtype, int rows_in_order, void* stream);
 // y [T, C] = exp(-exp(tanh(a [T, R]) w2^T + w0 [C])), float32; w2 comes transposed, w2t [R, C].
 int holon_decay_lora(const float* a, const void* w2t, const float* w0, float* y, int tokens, int channels, int rank,
                      int dtype, void* stream);

@@ -14,19 +14,19 @@
 namespace {
 
 template <typename T>
-__global__ void causal_conv_kernel(const T* __restrict__ x, const T* __restrict__ w, const T* __restrict__ state,
+__global__ void causal_conv_kernel(const T* __restrict__ x, const T* __restrict__ w, T* __restrict__ state,
                                    T* __restrict__ y, const int32_t* __restrict__ slots,
                                    const int32_t* __restrict__ starts, const int32_t* __restrict__ query_start,
                                    const int32_t* __restrict__ token_row, int channels, int taps, int add_input,
-                                   int act) {
+                                   int act, int keep) {
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
   const int t = blockIdx.y;
   if (c >= channels) return;
-  const int b = token_row[t];
-  const int q0 = query_start[b];
+  const int b = keep ? t : token_row[t];               // keep: every row has one token, token t is row t
+  const int q0 = keep ? t : query_start[b];
   const int i = t - q0;
   const bool carried = starts[b] > 0;
-  const T* held = state + (int64_t)slots[b] * (taps - 1) * channels;
+  T* held = state + (int64_t)slots[b] * (taps - 1) * channels;
   float acc = 0.f;
   for (int j = 0; j < taps; ++j) {
     const int l = i - (taps - 1) + j;
@@ -38,6 +38,11 @@ __global__ void causal_conv_kernel(const T* __restrict__ x, const T* __restrict_
   if (add_input) acc += Elem<T>::load(x[(int64_t)t * channels + c]);
   if (act) acc = silu<T>(acc);
   y[(int64_t)t * channels + c] = Elem<T>::store(acc);
+  if (keep) {                  // the row's one token: this thread alone reads and writes its channel of the slot
+    for (int e = 0; e + 2 < taps; ++e)
+      held[(int64_t)e * channels + c] = carried ? held[(int64_t)(e + 1) * channels + c] : Elem<T>::store(0.f);
+    if (taps > 1) held[(int64_t)(taps - 2) * channels + c] = x[(int64_t)t * channels + c];
+  }
 }
 
 // After the filter has read the old inputs: the slot takes the row's last taps - 1 inputs, oldest first. A thread
@@ -503,20 +508,21 @@ __global__ void __launch_bounds__(256) gated_out_kernel(const float* __restrict_
 }
 
 template <typename T>
-__global__ void shift_mix_kernel(const T* __restrict__ x, const T* __restrict__ mu, const T* __restrict__ state,
+__global__ void shift_mix_kernel(const T* __restrict__ x, const T* __restrict__ mu, T* __restrict__ state,
                                  T* __restrict__ y, const int32_t* __restrict__ slots, const int32_t* __restrict__ starts,
                                  const int32_t* __restrict__ query_start, const int32_t* __restrict__ token_row,
-                                 int tokens, int width, int mixes) {
+                                 int tokens, int width, int mixes, int keep) {
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
   const int t = blockIdx.y;
   if (c >= width) return;
-  const int b = token_row[t];
+  const int b = keep ? t : token_row[t];               // keep: every row has one token, token t is row t
   float prev = 0.f;
-  if (t > query_start[b]) prev = Elem<T>::load(x[(int64_t)(t - 1) * width + c]);
+  if (!keep && t > query_start[b]) prev = Elem<T>::load(x[(int64_t)(t - 1) * width + c]);
   else if (starts[b] > 0) prev = Elem<T>::load(state[(int64_t)slots[b] * width + c]);
   const float cur = Elem<T>::load(x[(int64_t)t * width + c]);
   for (int s = 0; s < mixes; ++s)
     y[((int64_t)s * tokens + t) * width + c] = Elem<T>::store(cur + (prev - cur) * Elem<T>::load(mu[(int64_t)s * width + c]));
+  if (keep) state[(int64_t)slots[b] * width + c] = x[(int64_t)t * width + c];
 }
 
 template <typename T>
@@ -569,18 +575,20 @@ __global__ void __launch_bounds__(256) decay_lora_kernel(const float* __restrict
 extern "C" int holon_causal_conv(const void* x, const void* w, void* state, void* y, const int32_t* slots,
                                  const int32_t* starts, const int32_t* query_start, const int32_t* token_row,
                                  int tokens, int rows, int channels, int taps, int state_slots, int add_input, int act,
-                                 int dtype, void* stream) {
+                                 int dtype, int rows_in_order, void* stream) {
   HOLON_CHECK(tokens >= 0 && rows >= 0 && channels > 0 && taps >= 1 && taps <= 16 && state_slots > 0,
               "causal_conv: tokens=%d rows=%d channels=%d taps=%d", tokens, rows, channels, taps);
   HOLON_CHECK(tokens <= 65535 && rows <= 65535, "causal_conv: %d tokens in %d rows exceed one launch", tokens, rows);
   if (tokens == 0 || rows == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
   const dim3 block(256), grid_t((channels + 255) / 256, tokens), grid_b((channels + 255) / 256, rows);
-  BY_DTYPE(dtype, (causal_conv_kernel<T><<<grid_t, block, 0, s>>>((const T*)x, (const T*)w, (const T*)state, (T*)y, slots,
-                                                                  starts, query_start, token_row, channels, taps,
-                                                                  add_input, act)));
+  HOLON_CHECK(!rows_in_order || tokens == rows, "causal_conv: rows in order means one token a row, got %d in %d", tokens,
+              rows);
+  BY_DTYPE(dtype, (causal_conv_kernel<T><<<grid_t, block, 0, s>>>((const T*)x, (const T*)w, (T*)state, (T*)y, slots, starts,
+                                                                  query_start, token_row, channels, taps, add_input,
+                                                                  act, rows_in_order)));
   HOLON_LAUNCH_OK();
-  if (taps > 1) {
+  if (taps > 1 && !rows_in_order) {
     BY_DTYPE(dtype, (causal_conv_keep_kernel<T><<<grid_b, block, 0, s>>>((const T*)x, (T*)state, slots, starts,
                                                                          query_start, channels, taps)));
     HOLON_LAUNCH_OK();
@@ -720,16 +728,21 @@ extern "C" int holon_gated_out(const float* o, const void* gate, const void* wei
 
 extern "C" int holon_shift_mix(const void* x, const void* mu, void* state, void* y, const int32_t* slots,
                                const int32_t* starts, const int32_t* query_start, const int32_t* token_row, int tokens,
-                               int rows, int width, int mixes, int state_slots, int dtype, void* stream) {
+                               int rows, int width, int mixes, int state_slots, int dtype, int rows_in_order,
+                               void* stream) {
   HOLON_CHECK(tokens >= 0 && rows >= 0 && width > 0 && mixes > 0 && state_slots > 0, "shift_mix: tokens=%d width=%d",
               tokens, width);
   HOLON_CHECK(tokens <= 65535 && rows <= 65535, "shift_mix: %d tokens in %d rows exceed one launch", tokens, rows);
   if (tokens == 0 || rows == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
   const dim3 block(256), grid_t((width + 255) / 256, tokens), grid_b((width + 255) / 256, rows);
-  BY_DTYPE(dtype, (shift_mix_kernel<T><<<grid_t, block, 0, s>>>((const T*)x, (const T*)mu, (const T*)state, (T*)y, slots,
-                                                                starts, query_start, token_row, tokens, width, mixes)));
+  HOLON_CHECK(!rows_in_order || tokens == rows, "shift_mix: rows in order means one token a row, got %d in %d", tokens,
+              rows);
+  BY_DTYPE(dtype, (shift_mix_kernel<T><<<grid_t, block, 0, s>>>((const T*)x, (const T*)mu, (T*)state, (T*)y, slots, starts,
+                                                                query_start, token_row, tokens, width, mixes,
+                                                                rows_in_order)));
   HOLON_LAUNCH_OK();
+  if (rows_in_order) return 0;                           // the one kernel has kept each row's token
   BY_DTYPE(dtype, (shift_keep_kernel<T><<<grid_b, block, 0, s>>>((const T*)x, (T*)state, slots, query_start, width)));
   HOLON_LAUNCH_OK();
   return 0;

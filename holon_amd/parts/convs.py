@@ -17,9 +17,10 @@ _P, _I = ctypes.c_void_p, ctypes.c_int
 _DT = {torch.float32: 0, torch.bfloat16: 1}
 
 
-def causal_conv_plain(x, weight, state, slots, starts, query_start, token_row, n_rows, add_input, silu):
+def causal_conv_plain(x, weight, state, slots, starts, query_start, token_row, n_rows, add_input, silu, in_order=False):
     """x [T, C], weight [C, taps], state [S, taps - 1, C] (updated in place), rows as the step lists them
-    (slots/starts [B], query_start [B + 1]). float32 arithmetic, taps added oldest first, one rounding."""
+    (slots/starts [B], query_start [B + 1]). float32 arithmetic, taps added oldest first, one rounding. `in_order`:
+    every row has one token and token t is row t (a kernel may then do everything in one launch)."""
     taps = weight.shape[1]
     y = torch.empty_like(x)
     w = weight.float()
@@ -41,7 +42,8 @@ def causal_conv_plain(x, weight, state, slots, starts, query_start, token_row, n
     return y
 
 
-def _causal_conv_hip(launch, x, weight, state, slots, starts, query_start, token_row, n_rows, add_input, silu):
+def _causal_conv_hip(launch, x, weight, state, slots, starts, query_start, token_row, n_rows, add_input, silu,
+                     in_order=False):
     t, c = x.shape
     taps = weight.shape[1]
     if not (x.is_cuda and x.is_contiguous() and x.dtype in _DT and weight.dtype == x.dtype and weight.is_contiguous()
@@ -52,12 +54,12 @@ def _causal_conv_hip(launch, x, weight, state, slots, starts, query_start, token
     y = torch.empty_like(x)
     launch(x.data_ptr(), weight.data_ptr(), state.data_ptr(), y.data_ptr(), slots.data_ptr(), starts.data_ptr(),
            query_start.data_ptr(), token_row.data_ptr(), t, n_rows, c, taps, state.shape[0], int(add_input), int(silu),
-           _DT[x.dtype])
+           _DT[x.dtype], int(bool(in_order) and t == n_rows))
     return y
 
 
 register_kernel(KernelOp("causal_conv", causal_conv_plain, "holon_causal_conv",
-                         [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I], _causal_conv_hip))
+                         [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I], _causal_conv_hip))
 
 
 class CausalConv(Part):
@@ -79,6 +81,7 @@ class CausalConv(Part):
 
     def forward(self, x: torch.Tensor, step, site) -> torch.Tensor:
         return self.kernels.causal_conv(x, self.weight, site.slot_state[self.name], step.slots, step.starts,
-                                        step.query_start, step.token_row, step.n_rows, self.add_input, self.silu)
+                                        step.query_start, step.token_row, step.n_rows, self.add_input, self.silu,
+                                        step.rows.in_order)
 
     __call__ = forward

@@ -132,10 +132,10 @@ def _gated_out_hip(launch, o, gate, weight, per_head_weight, eps, out_dtype):
 
 
 # -- decayed key-value memory -------------------------------------------------------------------------------------------
-def shift_mix_plain(x, mu, state, slots, starts, query_start, token_row, n_rows):
+def shift_mix_plain(x, mu, state, slots, starts, query_start, token_row, n_rows, in_order=False):
     """x [T, W]; mu [n, W]; state [S, W]: the last row each request has seen (zeros before its first). ->
     [n, T, W], mix_s = x + (x' - x) * mu_s with x' the row of the token before (float32 inside, one rounding); the
-    state takes each request's last row."""
+    state takes each request's last row. `in_order`: every row has one token and token t is row t."""
     prev = torch.empty_like(x)
     slot_of, start_of, qs = _rows(slots, starts, query_start, n_rows)
     for b in range(n_rows):
@@ -147,14 +147,15 @@ def shift_mix_plain(x, mu, state, slots, starts, query_start, token_row, n_rows)
     return (xf[None] + (pf - xf)[None] * mu.float()[:, None, :]).to(x.dtype)
 
 
-def _shift_mix_hip(launch, x, mu, state, slots, starts, query_start, token_row, n_rows):
+def _shift_mix_hip(launch, x, mu, state, slots, starts, query_start, token_row, n_rows, in_order=False):
     t, w = x.shape
     _need(x.is_cuda and x.is_contiguous() and x.dtype in _DT and mu.is_contiguous() and mu.dtype == x.dtype
           and mu.shape[1] == w and state.is_contiguous() and state.dtype == x.dtype and state.shape[1] == w,
           "shift_mix: shapes do not fit")
     y = torch.empty((mu.shape[0], t, w), dtype=x.dtype, device=x.device)
     launch(x.data_ptr(), mu.data_ptr(), state.data_ptr(), y.data_ptr(), slots.data_ptr(), starts.data_ptr(),
-           query_start.data_ptr(), token_row.data_ptr(), t, n_rows, w, mu.shape[0], state.shape[0], _DT[x.dtype])
+           query_start.data_ptr(), token_row.data_ptr(), t, n_rows, w, mu.shape[0], state.shape[0], _DT[x.dtype],
+           int(bool(in_order) and t == n_rows))
     return y
 
 
@@ -242,7 +243,7 @@ register_kernel(KernelOp("delta_scan", delta_scan_plain, "holon_delta_scan",
 register_kernel(KernelOp("gated_out", gated_out_plain, "holon_gated_out", [_P, _P, _P, _P, _I, _I, _I, _I, _F, _I],
                          _gated_out_hip))
 register_kernel(KernelOp("shift_mix", shift_mix_plain, "holon_shift_mix",
-                         [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I], _shift_mix_hip))
+                         [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I], _shift_mix_hip))
 register_kernel(KernelOp("decay_lora", decay_lora_plain, "holon_decay_lora", [_P, _P, _P, _P, _I, _I, _I, _I],
                          _decay_lora_hip))
 register_kernel(KernelOp("memory_scan", memory_scan_plain, "holon_memory_scan",
@@ -358,7 +359,8 @@ class DecayMemory(Part):
     def forward(self, x: torch.Tensor, step, site) -> torch.Tensor:
         k = self.kernels
         rows = (step.slots, step.starts, step.query_start)
-        mixes = k.shift_mix(x, self.mu, site.slot_state[self.prefix + "shift"], *rows, step.token_row, step.n_rows)
+        mixes = k.shift_mix(x, self.mu, site.slot_state[self.prefix + "shift"], *rows, step.token_row, step.n_rows,
+                            step.rows.in_order)
         r, kk, v, gate = (getattr(self, nm)(mixes[i]) for i, nm in enumerate(("r", "k", "v", "g")))
         lora = k.linear(mixes[4], self.w1, torch.float32)
         decay = k.decay_lora(lora, self.w2t, self.w0)
