@@ -155,7 +155,8 @@ def design(a) -> int:
             item = 2 if a.dtype == "bfloat16" else 4
             weights = sum(getattr(o, n).numel() * getattr(o, n).element_size()
                           for path, o, n, _ in engine.model.named_params() if not path.startswith("embed."))
-            state = engine.cache.nbytes() // (batch + 1) if name == "tolurax" else 0   # slot state (read and written)
+            # what a request keeps in its slot (the recurrences' matrices, the filters' inputs): read and written a step
+            state = sum(t[0].numel() * t.element_size() for _, _, t in engine.cache.slot_states)
             times = []
             for _ in range(3):
                 engine.add(torch.randint(0, z["vocab"], (prompt,), generator=g).tolist(), greedy(1))
