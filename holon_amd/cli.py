@@ -150,7 +150,7 @@ def replay_main(argv: list[str]) -> int:
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="the most tokens live requests hold at any time (each rounded up to a multiple of 64)")
     ap.add_argument("--page-size", type=int, default=16)
-    ap.add_argument("--max-seqs", type=int, default=8)
+    ap.add_argument("--max-seqs", type=int, default=4, help="requests that may be live at a time (state slots)")
     a = ap.parse_args(argv)
     if a.max_tokens < 1 or a.page_size < 1 or 64 % a.page_size:
         ap.error("--max-tokens must be positive and --page-size must divide 64")

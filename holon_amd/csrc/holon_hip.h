@@ -208,9 +208,10 @@ int holon_memory_scan(const void* r, const void* k, const void* v, const float* 
                       float* out, const int32_t* slots, const int32_t* starts, const int32_t* query_start, int rows,
                       int heads, int dim, int state_slots, int dtype, int piece_tokens, int max_pieces,
                       const int32_t* piece_base, float* sloc, float* pw, void* stream);
-// y [T, H V] = o / sqrt(mean_V(o^2) + eps) * weight * silu(gate); weight [V], or [H V] with per_head.
+// y [T, H V] = o / sqrt(mean_V(o^2) + eps) * weight * act(gate); weight [V], or [H V] with per_head; act is silu, or
+// with plain_sigmoid the sigmoid alone; a token's H V gates start gate_stride values after the token before's.
 int holon_gated_out(const float* o, const void* gate, const void* weight, void* y, int tokens, int heads, int vdim,
-                    int per_head, float eps, int dtype, void* stream);
+                    int per_head, float eps, int dtype, int64_t gate_stride, int plain_sigmoid, void* stream);
 // y [mixes, T, W] = x + (x' - x) mu_s, x' the row of the token before (state [state_slots, W] for a row's first
 // token, zeros for a row that starts at 0); the state then takes each row's last x.
 int holon_shift_mix(const void* x, const void* mu, void* state, void* y, const int32_t* slots, const int32_t* starts,
@@ -224,7 +225,7 @@ int holon_decay_lora(const float* a, const void* w2t, const float* w0, float* y,
 int holon_head_prepare(const void* qkv, void* q_out, int tokens, int heads, int kv_heads, int dim, int vdim,
                        const void* q_weight, const void* k_weight, float eps, const float* table, int rot, int table_rows,
                        const int32_t* positions, void* pages, const int32_t* write_page, const int32_t* write_off,
-                       int page_size, int num_pages, int dtype, void* stream);
+                       int page_size, int num_pages, int dtype, const float* bias, void* stream);
 int holon_sigmoid_attention(const void* q, void* out, const void* pages, const int32_t* table, int table_stride,
                             const int32_t* slots, const int32_t* token_row, const int32_t* positions,
                             const int32_t* query_start, const int32_t* row_ids, int tokens, int heads, int kv_heads,
@@ -242,6 +243,30 @@ int holon_sigmoid_attention_decode_bf16(const void* q, void* out, const void* pa
                                         const int32_t* query_start, const int32_t* row_ids, int n_rows, int max_len,
                                         int heads, int kv_heads, int head_dim, int page_size, float scale, int window,
                                         const float* head_bias, const void* gate, int rows_in_order, void* stream);
+
+// -- Dynamic Tanh and the adds around it (dyt.hip) ------------------------------------------------------------------------
+// x [rows, dim] (float32 when anything is added): x += scale * (tanh(a1 term) w1 + b1) (with a term), x += extra (with
+// extra, float32), y = tanh(a2 x) w2 + b2 (with y); the alphas are single values on the device, w and b [dim] float32.
+int holon_dyt_stream(void* x, int x_dtype, const void* term, int term_dtype, const float* post_alpha,
+                     const float* post_w, const float* post_b, float scale, const float* extra, const float* pre_alpha,
+                     const float* pre_w, const float* pre_b, void* y, int y_dtype, int64_t rows, int dim, void* stream);
+
+// -- softmax attention with a window and a sink over pages of keys [Hkv, P, D] then values [Hkv, V, P] ------------------
+// (softmax_attention.hip) q [T, H, D] -> out [T, H V]; token t reads block table row slots[token_row[t]] and stands at
+// positions[t]; sink [H] float32 or null; window 0: everything before.
+int holon_softmax_attention(const void* q, void* out, const void* pages, const int32_t* table, int table_stride,
+                            int table_rows, const int32_t* slots, const int32_t* token_row, const int32_t* positions,
+                            int tokens, int heads, int kv_heads, int dim, int vdim, int page_size, int num_pages,
+                            const float* sink, float scale, int window, int dtype, void* stream);
+
+// -- the matrix memory of xLSTM (mlstm.hip) -------------------------------------------------------------------------------
+// proj [T, width]: q, k [H D] and v [H V] and the gates' pre-activations [2 H] (input, then forget) from the given
+// columns; gate_bias [2 H]; state S [slots, H, D, V], n [slots, H, ceil(V / 8), D], m [slots, H, ceil(V / 8)] (a copy
+// for every 8 value columns), float32; out [T, H, V] float32.
+int holon_mlstm_scan(const void* proj, int width, int q_off, int k_off, int v_off, int gate_off, const float* gate_bias,
+                     float cap, float* S, float* n, float* m, float* out, const int32_t* slots, const int32_t* starts,
+                     const int32_t* query_start, int rows, int heads, int dim, int vdim, int state_slots, int dtype,
+                     void* stream);
 
 #ifdef __cplusplus
 }

@@ -15,8 +15,9 @@
 
 namespace {
 
-// One wave per (token, head of q, k or v). q and k: x * rsqrt(mean(x^2) + eps) * weight (if weights), then the
-// half-split rotation of the first `rot` dimensions; one rounding.
+// One wave per (token, head of q, k or v). `bias` (one float32 a column of the projection, or null) is added first. q and
+// k: x * rsqrt(mean(x^2) + eps) * weight (if weights), then the half-split rotation of the first `rot` dimensions; one
+// rounding.
 template <typename T>
 __global__ void __launch_bounds__(256) head_prepare_kernel(const T* __restrict__ qkv, T* __restrict__ q_out, int heads,
                                                            int kv_heads, int dim, int vdim,
@@ -25,7 +26,7 @@ __global__ void __launch_bounds__(256) head_prepare_kernel(const T* __restrict__
                                                            int table_rows, const int32_t* __restrict__ positions,
                                                            T* __restrict__ pages, const int32_t* __restrict__ write_page,
                                                            const int32_t* __restrict__ write_off, int page_size,
-                                                           int num_pages) {
+                                                           int num_pages, const float* __restrict__ bias) {
   const int t = blockIdx.x;
   const int hs = blockIdx.y * 4 + threadIdx.x / WAVE;
   const int lane = threadIdx.x % WAVE;
@@ -38,9 +39,15 @@ __global__ void __launch_bounds__(256) head_prepare_kernel(const T* __restrict__
   if (hs >= heads + kv_heads) {                       // a value head: stored as it is
     const int hv = hs - heads - kv_heads;
     if (!page_ok) return;
-    const T* src = row + (int64_t)(heads + kv_heads) * dim + (int64_t)hv * vdim;
+    const int64_t col = (int64_t)(heads + kv_heads) * dim + (int64_t)hv * vdim;
+    const T* src = row + col;
     T* dst = pages + page * page_len + (int64_t)kv_heads * page_size * dim + (int64_t)hv * vdim * page_size + off;
-    for (int d = lane; d < vdim; d += WAVE) dst[(int64_t)d * page_size] = src[d];
+    if (bias) {
+      for (int d = lane; d < vdim; d += WAVE)
+        dst[(int64_t)d * page_size] = Elem<T>::store(Elem<T>::load(src[d]) + bias[col + d]);
+    } else {
+      for (int d = lane; d < vdim; d += WAVE) dst[(int64_t)d * page_size] = src[d];
+    }
     return;
   }
   const bool is_q = hs < heads;
@@ -49,11 +56,13 @@ __global__ void __launch_bounds__(256) head_prepare_kernel(const T* __restrict__
   T* dst = is_q ? q_out + ((int64_t)t * heads + hs) * dim
                 : pages + page * page_len + ((int64_t)(hs - heads) * page_size + off) * dim;
   const T* w = is_q ? q_weight : k_weight;
+  const float* bs = bias ? bias + (int64_t)hs * dim : nullptr;
+  auto in = [&](int d) { return Elem<T>::load(src[d]) + (bs ? bs[d] : 0.f); };
   float r = 1.f;
   if (w) {
     float ss = 0.f;
     for (int d = lane; d < dim; d += WAVE) {
-      const float v = Elem<T>::load(src[d]);
+      const float v = in(d);
       ss += v * v;
     }
     r = 1.0f / sqrtf(wave_sum(ss) / (float)dim + eps);
@@ -64,15 +73,15 @@ __global__ void __launch_bounds__(256) head_prepare_kernel(const T* __restrict__
     pos = pos < 0 ? 0 : (pos >= table_rows ? table_rows - 1 : pos);
     const float* cs = table + (int64_t)pos * rot;
     for (int p = lane; p < half; p += WAVE) {
-      const float a = Elem<T>::load(src[p]) * r * (w ? Elem<T>::load(w[p]) : 1.f);
-      const float b = Elem<T>::load(src[p + half]) * r * (w ? Elem<T>::load(w[p + half]) : 1.f);
+      const float a = in(p) * r * (w ? Elem<T>::load(w[p]) : 1.f);
+      const float b = in(p + half) * r * (w ? Elem<T>::load(w[p + half]) : 1.f);
       const float c = cs[p], s = cs[half + p];
       dst[p] = Elem<T>::store(a * c - b * s);
       dst[p + half] = Elem<T>::store(b * c + a * s);
     }
   }
   for (int d = (table ? rot : 0) + lane; d < dim; d += WAVE)
-    dst[d] = Elem<T>::store(Elem<T>::load(src[d]) * r * (w ? Elem<T>::load(w[d]) : 1.f));
+    dst[d] = Elem<T>::store(in(d) * r * (w ? Elem<T>::load(w[d]) : 1.f));
 }
 
 // The general kernel (any dtype and sizes; the decode rows of every step): one block of four waves per (token, head).
@@ -165,7 +174,8 @@ __global__ void __launch_bounds__(256) sigmoid_attention_kernel(const T* __restr
 extern "C" int holon_head_prepare(const void* qkv, void* q_out, int tokens, int heads, int kv_heads, int dim, int vdim,
                                   const void* q_weight, const void* k_weight, float eps, const float* table, int rot,
                                   int table_rows, const int32_t* positions, void* pages, const int32_t* write_page,
-                                  const int32_t* write_off, int page_size, int num_pages, int dtype, void* stream) {
+                                  const int32_t* write_off, int page_size, int num_pages, int dtype, const float* bias,
+                                  void* stream) {
   HOLON_CHECK(tokens >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dim > 0 && vdim > 0,
               "head_prepare: %d/%d heads of %d/%d", heads, kv_heads, dim, vdim);
   HOLON_CHECK((table == nullptr && rot == 0) || (rot > 0 && rot % 2 == 0 && rot <= dim && table_rows > 0),
@@ -180,12 +190,12 @@ extern "C" int holon_head_prepare(const void* qkv, void* q_out, int tokens, int 
     head_prepare_kernel<float><<<grid, 256, 0, s>>>((const float*)qkv, (float*)q_out, heads, kv_heads, dim, vdim,
                                                     (const float*)q_weight, (const float*)k_weight, eps, table, rot,
                                                     table_rows, positions, (float*)pages, write_page, write_off,
-                                                    page_size, num_pages);
+                                                    page_size, num_pages, bias);
   else
     head_prepare_kernel<bf16_t><<<grid, 256, 0, s>>>((const bf16_t*)qkv, (bf16_t*)q_out, heads, kv_heads, dim, vdim,
                                                      (const bf16_t*)q_weight, (const bf16_t*)k_weight, eps, table, rot,
                                                      table_rows, positions, (bf16_t*)pages, write_page, write_off,
-                                                     page_size, num_pages);
+                                                     page_size, num_pages, bias);
   HOLON_LAUNCH_OK();
   return 0;
 }

@@ -29,6 +29,7 @@ class Site:
     layer: int
     writes: bool = True
     owner: int | None = None                      # the run whose cache this one reads (None: its own)
+    turn: int = 0                                 # how many earlier runs were of the same layer (a looped layer's pass)
     group: int | None = None                      # paged group id
     pages: torch.Tensor | None = None             # this site's page storage [num_pages, P * elems]
     paged: dict[str, SitePages] = dataclasses.field(default_factory=dict)
@@ -54,7 +55,8 @@ class Model(Part):
         self.attach("norm", build.make(spec.norm, dim=spec.hidden))
         self.attach("lm_head", build.make(spec.head, vocab=spec.vocab, hidden=spec.hidden, embed=self.embed))
         self._keeps_origin = any(b.reads_origin for b in self.blocks)
-        self.sites = [Site(run=at, layer=r.layer, writes=r.reads is None, owner=r.reads)
+        self.sites = [Site(run=at, layer=r.layer, writes=r.reads is None, owner=r.reads,
+                           turn=sum(1 for before in spec.order[:at] if before.layer == r.layer))
                       for at, r in enumerate(spec.order)]
 
     def state_decls(self) -> list[list[PagedState | SlotState]]:

@@ -7,12 +7,16 @@ from .ffn import SwiGLU
 from .linear import Linear
 from .mixers import GQA, ParallelMixers
 from .norms import Normed, RMSNorm
-from .positions import BandedRope, NoPosition, Rope, rope_table
+from .positions import BandedRope, NoPosition, Rope, YarnRope, rope_table
 from .convs import CausalConv
 from .recurrent import DecayMemory, GatedDelta
 from .sigmoid_attention import SigmoidWindowAttention
 from .stream32 import LayerNorm, Pending, PreNorm32
+from .dyt import DynamicTanh, Sandwich32, Scaled
+from .softmax_attention import LatentAttention, SoftmaxAttention
+from .mlstm import MLSTM
 
 __all__ = ["FLOAT32", "INT32", "MODEL", "Build", "EmbedPart", "NormPart", "PagedState", "ParamDecl", "Part", "PartialSums", "SlotState", "Stream", "PreNorm",
            "Embedding", "LMHead", "SwiGLU", "Linear", "GQA", "Normed", "RMSNorm", "NoPosition", "Rope", "rope_table", "BandedRope", "CausalConv", "DecayMemory", "GatedDelta",
-           "SigmoidWindowAttention", "LayerNorm", "Pending", "PreNorm32", "ParallelMixers"]
+           "SigmoidWindowAttention", "LayerNorm", "Pending", "PreNorm32", "ParallelMixers",
+           "DynamicTanh", "Sandwich32", "Scaled", "LatentAttention", "SoftmaxAttention", "MLSTM", "YarnRope"]

@@ -4,16 +4,23 @@ from __future__ import annotations
 import torch
 
 from ..registry import register_part
+from ..spec import PartRef
 from .base import Build, EmbedPart, Part
 
 
 @register_part("embed", "table")
 class Embedding(EmbedPart):
+    """Rows of a table. With `norm` (any registered norm whose `forward` takes `out_dtype`) the rows go through it
+    and come out in float32: the start of a residual stream that is kept in 32-bit."""
+
     graph_safe = True
 
-    def __init__(self, build: Build, *, vocab: int, hidden: int) -> None:
+    def __init__(self, build: Build, *, vocab: int, hidden: int, norm: PartRef | None = None) -> None:
         super().__init__(build)
         self.declare("weight", (vocab, hidden))
+        self.norm = None
+        if norm is not None:
+            self.attach("norm", build.make(norm, dim=hidden))
 
     def rows(self, ids: torch.Tensor) -> torch.Tensor:
         return self.kernels.embedding(ids, self.weight)
@@ -22,7 +29,10 @@ class Embedding(EmbedPart):
                 want_stats: bool = False):
         """Rows of the table; `take`: where a token is still on the device, see the kernel contract. With
         `want_stats`: (rows, their statistics for a norm that follows, or None)."""
-        return self.kernels.embedding(ids, self.weight, take, want_stats)
+        if self.norm is None:
+            return self.kernels.embedding(ids, self.weight, take, want_stats)
+        rows = self.norm(self.kernels.embedding(ids, self.weight, take, False), out_dtype=torch.float32)
+        return (rows, None) if want_stats else rows
 
     __call__ = forward
 

@@ -81,6 +81,52 @@ class BandedRope(Rope):
         self.table = torch.cat((angles.cos(), angles.sin()), dim=-1).contiguous().to(build.device)
 
 
+def yarn_frequencies(rotary_dim: int, base: float, scaling: dict | None) -> tuple[torch.Tensor, float]:
+    """(f_i for the rotary_dim/2 pairs as float32, computed in float64 and rounded once; the factor both cos and sin
+    are multiplied by). Plain: f_i = base^(-2i/rotary_dim), factor 1. With `scaling` = {factor, original, fast, slow}
+    (YaRN): the pair that turns t times over `original` positions has index d(t) = rotary_dim ln(original / (2 pi t))
+    / (2 ln base); pairs up to lo = max(floor(d(fast)), 0) keep f_i, pairs from hi = min(ceil(d(slow)),
+    rotary_dim - 1) on turn `factor` times slower, and between them the two are blended linearly in the index
+    (ramp = clamp((i - lo) / max(hi - lo, 0.001), 0, 1)); cos and sin are multiplied by 0.1 ln(factor) + 1."""
+    i = torch.arange(rotary_dim // 2, dtype=torch.float64)
+    f = torch.as_tensor(float(base), dtype=torch.float64) ** (-2.0 * i / rotary_dim)
+    if not scaling:
+        return f.to(torch.float32), 1.0
+    factor, original, fast, slow = (float(scaling[k]) for k in ("factor", "original", "fast", "slow"))
+
+    def index_of(turns: float) -> float:
+        return rotary_dim * math.log(original / (2 * math.pi * turns)) / (2 * math.log(base))
+    lo = max(math.floor(index_of(fast)), 0)
+    hi = min(math.ceil(index_of(slow)), rotary_dim - 1)
+    ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0, 1)
+    return (f / factor * ramp + f * (1 - ramp)).to(torch.float32), 0.1 * math.log(factor) + 1.0
+
+
+@register_part("position", "rope_yarn")
+class YarnRope(Rope):
+    """Rotary embedding on the first `rotary_dim` dimensions of a head with YaRN's rescaling of the frequencies
+    (`scaling`, a dict or its sorted items; None: plain frequencies). `interleaved` says that the design pairs
+    dimensions (2i, 2i + 1); the table is laid out for the kernels' half-split pairing all the same, and a mixer that
+    sees `interleaved` reorders its q and k projections' rows to match (every score stays what it was). Angles are the
+    float32 product of position and frequency."""
+
+    graph_safe = True
+
+    def __init__(self, build: Build, *, theta: float, head_dim: int, rotary_dim: int | None = None, scaling=None,
+                 interleaved: bool = False) -> None:
+        Part.__init__(self, build)
+        self.theta, self.head_dim = float(theta), head_dim
+        self.rotary_dim = head_dim if rotary_dim is None else int(rotary_dim)
+        if self.rotary_dim % 2 or not 0 < self.rotary_dim <= head_dim:
+            raise ValueError(f"rotary_dim {self.rotary_dim} must be even and within head_dim {head_dim}")
+        self.scaling = dict(scaling) if scaling else None
+        self.interleaved = bool(interleaved)
+        freqs, gain = yarn_frequencies(self.rotary_dim, self.theta, self.scaling)
+        angles = torch.arange(build.max_model_len, dtype=torch.float32)[:, None] * freqs[None, :]
+        gain = torch.tensor(gain, dtype=torch.float32)
+        self.table = torch.cat((angles.cos() * gain, angles.sin() * gain), dim=-1).contiguous().to(build.device)
+
+
 @register_part("position", "none")
 class NoPosition(Part):
     """No position encoding (order enters through the causal mask alone)."""

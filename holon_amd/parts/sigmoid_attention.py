@@ -28,16 +28,19 @@ def _ptr(t):
 
 
 def head_prepare_plain(qkv, heads, kv_heads, dim, vdim, q_weight, k_weight, eps, table, positions, pages, write_page,
-                       write_off, page_size):
-    """qkv [T, (H + G) D + G V] (queries, keys, values side by side). Per head of q and k: x * rsqrt(mean(x^2) + eps)
+                       write_off, page_size, bias=None):
+    """qkv [T, (H + G) D + G V] (queries, keys, values side by side); `bias` (float32, one value a column, or None)
+    is added first. Per head of q and k: x * rsqrt(mean(x^2) + eps)
     * weight (when weights are given), then the rotation by `table` [positions, rot] (cos of rot/2 angles, then
     their sines; pairs (i, i + rot/2); dimensions from rot on pass), all in float32 with one rounding. Keys and
     values go into `pages` [pages, G P (D + V)] (keys [G, P, D], then values [G, V, P]) at (write_page[t],
     write_off[t]); returns q [T, H, D]."""
     t = qkv.shape[0]
+    if bias is not None:
+        qkv = qkv.float() + bias.float()
     q = qkv[:, : heads * dim].float().view(t, heads, dim)
     k = qkv[:, heads * dim: (heads + kv_heads) * dim].float().view(t, kv_heads, dim)
-    v = qkv[:, (heads + kv_heads) * dim:].view(t, kv_heads, vdim)
+    v = qkv[:, (heads + kv_heads) * dim:].reshape(t, kv_heads, vdim)
     if q_weight is not None:
         q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + eps) * q_weight.float()
         k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + eps) * k_weight.float()
@@ -54,11 +57,11 @@ def head_prepare_plain(qkv, heads, kv_heads, dim, vdim, q_weight, k_weight, eps,
     vals = pages[:, kv_heads * page_size * dim:].view(-1, kv_heads, vdim, page_size)
     keys[write_page.long(), :, write_off.long()] = k.to(pages.dtype)
     vals[write_page.long(), :, :, write_off.long()] = v.to(pages.dtype)
-    return q.to(qkv.dtype)
+    return q.to(pages.dtype)
 
 
 def _head_prepare_hip(launch, qkv, heads, kv_heads, dim, vdim, q_weight, k_weight, eps, table, positions, pages,
-                      write_page, write_off, page_size):
+                      write_page, write_off, page_size, bias=None):
     t, width = qkv.shape
     ok = qkv.is_cuda and qkv.is_contiguous() and qkv.dtype in _DT and width == (heads + kv_heads) * dim + kv_heads * vdim \
         and pages.dtype == qkv.dtype and pages.is_contiguous() and pages.dim() == 2 \
@@ -66,7 +69,8 @@ def _head_prepare_hip(launch, qkv, heads, kv_heads, dim, vdim, q_weight, k_weigh
         and all(w is None or (w.dtype == qkv.dtype and w.shape == (dim,)) for w in (q_weight, k_weight)) \
         and (table is None or (table.dtype == torch.float32 and table.is_contiguous() and table.shape[1] % 2 == 0
                                and table.shape[1] <= dim)) \
-        and write_page.shape[0] >= t and write_off.shape[0] >= t and positions.shape[0] >= t
+        and write_page.shape[0] >= t and write_off.shape[0] >= t and positions.shape[0] >= t \
+        and (bias is None or (bias.dtype == torch.float32 and bias.is_contiguous() and bias.shape == (width,)))
     if not ok:
         raise ValueError(f"head_prepare: qkv {tuple(qkv.shape)} {qkv.dtype}, pages {tuple(pages.shape)} do not fit "
                          f"{heads}/{kv_heads} heads of {dim}/{vdim}, page {page_size}")
@@ -74,7 +78,7 @@ def _head_prepare_hip(launch, qkv, heads, kv_heads, dim, vdim, q_weight, k_weigh
     launch(qkv.data_ptr(), q.data_ptr(), t, heads, kv_heads, dim, vdim, _ptr(q_weight), _ptr(k_weight), float(eps),
            _ptr(table), table.shape[1] if table is not None else 0, table.shape[0] if table is not None else 0,
            positions.data_ptr(), pages.data_ptr(), write_page.data_ptr(), write_off.data_ptr(), page_size,
-           pages.shape[0], _DT[qkv.dtype])
+           pages.shape[0], _DT[qkv.dtype], _ptr(bias))
     return q
 
 
@@ -143,7 +147,7 @@ def _sigmoid_attention_hip(launch, q, pages, table, rows, token_row, positions, 
 
 
 register_kernel(KernelOp("head_prepare", head_prepare_plain, "holon_head_prepare",
-                         [_P, _P, _I, _I, _I, _I, _I, _P, _P, _F, _P, _I, _I, _P, _P, _P, _P, _I, _I, _I],
+                         [_P, _P, _I, _I, _I, _I, _I, _P, _P, _F, _P, _I, _I, _P, _P, _P, _P, _I, _I, _I, _P],
                          _head_prepare_hip))
 register_kernel(KernelOp("sigmoid_attention", sigmoid_attention_plain,
                          ("holon_sigmoid_attention", "holon_sigmoid_attention_prefill_bf16",
