@@ -21,7 +21,7 @@ The engine is one process on one GPU; for --gpus > 1 a line says so and the exit
 prompt tokens at the Qwen3-32B shape, portions of 512 tokens beside decode rows, 256 greedy tokens each; `long` is 8
 prompts of 32,768 tokens at the Qwen3-4B shape, 512 tokens each at temperature 0.7.
 
---workload tolurax measures the Tolurax design beside Qwen3 at equal sizes (width, layers, heads, head size,
+--workload tolurax (or relanex) measures that design beside Qwen3 at equal sizes (width, layers, heads, head size,
 feed-forward, vocabulary; random weights): a 2,048-token prompt and decode at batch 8 near a context of 2,048, at two
 sizes (`--sizes`), one line with both models' figures and the bytes a decode step must read. `--only` runs one model
 (for a profiler).
@@ -124,6 +124,44 @@ def tolurax_config(z: dict, window: int = 1024) -> dict:
             "canon": {"taps": 3}, "logit_softcap": 30.0, "layers": [layer(i) for i in range(z["layers"])]}
 
 
+def relanex_config(z: dict, window: int = 1024) -> dict:
+    """A Relanex model of a size's layers, in fours: softmax attention with the size's heads (half of each head
+    rotated, YaRN), two latent-attention layers (the size's heads, latents of 768 and 256, a window), and a matrix
+    memory with heads of 128, a feed-forward in each."""
+    def layer(i: int) -> dict:
+        mlp = {"kind": "dense", "ff": z["ff"]}
+        if i % 4 == 0:
+            return {"type": "attention", "mlp": mlp,
+                    "mixer": {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["dim"],
+                              "scale": z["dim"] ** -0.5,
+                              "rot": {"dims": z["dim"] // 2, "base": 250000.0,
+                                      "scaling": {"factor": 4.0, "original": 2048, "fast": 32.0, "slow": 1.0}}}}
+        if i % 4 == 3:
+            return {"type": "mlstm", "mlp": mlp, "mixer": {"heads": z["width"] // 128, "dim": 128, "vdim": 128,
+                                                          "gate_cap": 15.0}}
+        return {"type": "latent_attention", "mlp": mlp,
+                "mixer": {"heads": z["heads"], "dim": z["dim"], "vdim": z["dim"], "q_rank": 768, "kv_rank": 256,
+                          "mask": {"size": window}, "scale": z["dim"] ** -0.5}}
+    return {"architecture": "Relanex", "width": z["width"], "vocab": z["vocab"], "norm": {"eps": 1e-6},
+            "residual_mult": 0.7, "layers": [layer(i) for i in range(z["layers"])]}
+
+
+def design_cache_bytes(name: str, cfg_json: dict, z: dict, item: int, batch: int, context: int) -> int:
+    """The bytes of paged cache a decode step of `batch` rows near `context` reads."""
+    if name == "qwen3":
+        return z["layers"] * 2 * z["kv_heads"] * z["dim"] * item * batch * context
+    total = 0
+    for layer in cfg_json["layers"]:
+        m = layer["mixer"]
+        if layer["type"] == "parallel":             # the window's keys and values
+            total += 2 * z["kv_heads"] * z["dim"] * item * batch * min(context, m["left"]["mask"]["size"])
+        elif layer["type"] == "attention":
+            total += m["kv_heads"] * (m["dim"] + m["vdim"]) * item * batch * context
+        elif layer["type"] == "latent_attention":   # the latent, held as keys and as values
+            total += 2 * m["kv_rank"] * item * batch * min(context, m["mask"]["size"])
+    return total
+
+
 def qwen3_config(z: dict) -> dict:
     return {"architectures": ["Qwen3ForCausalLM"], "num_hidden_layers": z["layers"], "hidden_size": z["width"],
             "num_attention_heads": z["heads"], "num_key_value_heads": z["kv_heads"], "head_dim": z["dim"],
@@ -132,7 +170,7 @@ def qwen3_config(z: dict) -> dict:
 
 
 def design(a) -> int:
-    """Tolurax beside Qwen3 at equal sizes: prompt and decode throughput, one line."""
+    """A design (Tolurax or Relanex) beside Qwen3 at equal sizes: prompt and decode throughput, one line."""
     import gc
 
     import torch
@@ -145,7 +183,8 @@ def design(a) -> int:
     out: dict = {}
     for size in a.sizes.split(","):
         z = DESIGN_SIZES[size]
-        for name, cfg_json in (("tolurax", tolurax_config(z)), ("qwen3", qwen3_config(z))):
+        ours = tolurax_config(z) if a.workload == "tolurax" else relanex_config(z)
+        for name, cfg_json in ((a.workload, ours), ("qwen3", qwen3_config(z))):
             if a.only and a.only != name:
                 continue
             engine = Engine.from_random(cfg_json, seed=0, cfg=EngineConfig(
@@ -182,10 +221,7 @@ def design(a) -> int:
             ms = (time.perf_counter() - t0) * 1e3 / a.steps
             while engine.has_work():
                 engine.step()
-            kv = 0 if name == "tolurax" else z["layers"] * 2 * z["kv_heads"] * z["dim"] * item * batch * context
-            if name == "tolurax":           # the window's keys and values of the parallel layers
-                kv = sum(2 * z["kv_heads"] * z["dim"] * item * batch * min(context, 1024)
-                         for layer in cfg_json["layers"] if layer["type"] == "parallel")
+            kv = design_cache_bytes(name, cfg_json, z, item, batch, context)
             step_gb = (weights + kv + 2 * state * batch) / 1e9
             out.setdefault(size, {})[name] = {
                 "prefill_tokens_per_s": round(prompt / (min(times) * 1e-3), 1), "prefill_ms": round(min(times), 3),
@@ -197,7 +233,8 @@ def design(a) -> int:
             del engine
             gc.collect()
             torch.cuda.empty_cache()
-    print(json.dumps({"metric": "Tolurax beside Qwen3 at equal sizes: 2,048-token prompt, decode at batch 8 near context 2,048",
+    print(json.dumps({"metric": f"{a.workload.capitalize()} beside Qwen3 at equal sizes: 2,048-token prompt, decode at batch 8 near "
+                                "context 2,048",
                       "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
                       "dtype": "bf16" if a.dtype == "bfloat16" else "fp32",
                       "data": "synthetic (random weights, uniform random token ids)",
@@ -219,9 +256,10 @@ def main(argv: list[str] | None = None) -> int:
     ap.add_argument("--context", type=int, default=CONTEXT, help="the context the timed decode steps end at")
     ap.add_argument("--prompt", type=int, default=PROMPT, help="tokens of the timed prompt")
     ap.add_argument("--no-graphs", action="store_true")
-    ap.add_argument("--workload", choices=("decode", "mixed", "long", "tolurax"), default="decode")
-    ap.add_argument("--sizes", default="2k,4k", help="--workload tolurax: which of its sizes (2k, 4k) to run")
-    ap.add_argument("--only", choices=("tolurax", "qwen3"), default=None, help="--workload tolurax: one model only")
+    ap.add_argument("--workload", choices=("decode", "mixed", "long", "tolurax", "relanex"), default="decode")
+    ap.add_argument("--sizes", default="2k,4k", help="--workload tolurax|relanex: which of its sizes (2k, 4k) to run")
+    ap.add_argument("--only", choices=("tolurax", "relanex", "qwen3"), default=None,
+                    help="--workload tolurax|relanex: one model only")
     ap.add_argument("--products", choices=("own", "vendor", "timed"), default="timed",
                     help="EngineConfig.products: which kernel products of 17 to 1,024 rows take (reported in the line)")
     a = ap.parse_args(argv)
@@ -232,7 +270,7 @@ def main(argv: list[str] | None = None) -> int:
         from .kernels import build as kernel_build
         if kernel_build.find_library() is None:
             kernel_build.build()
-        if a.workload == "tolurax":
+        if a.workload in ("tolurax", "relanex"):
             return design(a)
         return workload(a.workload, None if "--layers" not in (argv or sys.argv) else a.layers, a.dtype, a.products)
 

@@ -62,7 +62,17 @@ struct AttnArgs {
   float scale;
   const float* head_bias;
   const bf16_t* gate;
+  // softmax with a sink (nullable, [Hq], in the scores' natural units): exp(sink[head] - max) joins the denominator;
+  // it has no key and no value
+  const float* sink;
 };
+
+// The denominator of a row whose keys summed to `l` under the running maximum `m` (in units of log2): with a sink, its
+// term beside them. A row that saw no key (m = -inf) keeps l = 0 and its result of zero.
+__device__ __forceinline__ float with_sink(const AttnArgs& a, int head, float l, float m) {
+  if (a.sink == nullptr || m == -INFINITY) return l;
+  return l + exp2f(a.sink[head] * 1.4426950408889634f - m);
+}
 
 // How the 16 rows of a tile map to (position, head) for a group of G heads.
 struct TileMap {
@@ -356,6 +366,7 @@ __global__ void __launch_bounds__(256) attn_prefill_kernel(AttnArgs a) {
     lt += __shfl_xor(lt, 16, WAVE);
     lt += __shfl_xor(lt, 32, WAVE);
     if (!rr[t].valid) continue;
+    lt = with_sink(a, rr[t].head, lt, m[t]);
     const float inv = lt > 0.f ? 1.0f / lt : 0.f;
     bf16_t* op = a.out + ((int64_t)rr[t].token * a.heads + rr[t].head) * D + 4 * g;
 #pragma unroll
@@ -561,6 +572,7 @@ __global__ void __launch_bounds__(256) attn_prefill_lds_kernel(AttnArgs a) {
       lt += __shfl_xor(lt, 16, WAVE);
       lt += __shfl_xor(lt, 32, WAVE);
       if (!rr[t].valid) continue;
+      lt = with_sink(a, rr[t].head, lt, m[t]);
       const float inv = lt > 0.f ? 1.0f / lt : 0.f;
       bf16_t* op = a.out + ((int64_t)rr[t].token * a.heads + rr[t].head) * D + 4 * g;
 #pragma unroll
@@ -832,6 +844,7 @@ __global__ void __launch_bounds__(256, D == 128 ? 2 : 3) attn_prefill_wide_kerne
     }
     float lt = l + __shfl_xor(l, 32, WAVE);
     if (valid) {
+      if (!SIG) lt = with_sink(a, head, lt, m);
       const float inv = SIG ? 1.0f : (lt > 0.f ? 1.0f / lt : 0.f);
       bf16_t* op = a.out + ((int64_t)token * a.heads + head) * D + 4 * h;
       const bf16_t* gp = SIG && a.gate ? a.gate + ((int64_t)token * a.heads + head) * D + 4 * h : nullptr;
@@ -1126,6 +1139,7 @@ __global__ void __launch_bounds__(256, 2) attn_prefill_dma_kernel(AttnArgs a) {
     stage(std::true_type{}, kb_last, buf);
     float lt = l + __shfl_xor(l, 32, WAVE);
     if (valid) {
+      lt = with_sink(a, head, lt, m);
       const float inv = lt > 0.f ? 1.0f / lt : 0.f;
       bf16_t* op = a.out + ((int64_t)token * a.heads + head) * D + 4 * h;
 #pragma unroll
@@ -1370,8 +1384,9 @@ __global__ void __launch_bounds__(256, 1) attn_prefill_pair_kernel(AttnArgs a) {
     }
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
-      const float lt = l[t] + __shfl_xor(l[t], 32, WAVE);
+      float lt = l[t] + __shfl_xor(l[t], 32, WAVE);
       if (valid[t]) {
+        lt = with_sink(a, head, lt, m[t]);
         const float inv = lt > 0.f ? 1.0f / lt : 0.f;
         bf16_t* op = a.out + ((int64_t)token[t] * a.heads + head) * D + 4 * h;
 #pragma unroll
@@ -1641,6 +1656,7 @@ __global__ void __launch_bounds__(512) attn_decode_kernel(AttnArgs a, FusedArgs 
   }
   if (wave == 0 && rr.valid) {
     if (a.out_splits == 1) {             // the row's whole result: normalised and rounded here
+      if (!SIG) lt = with_sink(a, rr.head, lt, mt);
       const float inv = SIG ? 1.0f : (lt > 0.f ? 1.0f / lt : 0.f);
       bf16_t* op = a.out + ((int64_t)rr.token * a.heads + rr.head) * D + 4 * g;
       const bf16_t* gp = SIG && a.gate ? a.gate + ((int64_t)rr.token * a.heads + rr.head) * D + 4 * g : nullptr;
@@ -1682,7 +1698,8 @@ template <int D>
 __global__ void __launch_bounds__(256) attn_merge_kernel(const float* __restrict__ part_o,
                                                          const float* __restrict__ part_ml, bf16_t* __restrict__ out,
                                                          const int32_t* __restrict__ row_ids,
-                                                         const int32_t* __restrict__ qstart, int heads, int splits) {
+                                                         const int32_t* __restrict__ qstart, int heads, int splits,
+                                                         const float* __restrict__ sink) {
   constexpr int LANES = D / 4;            // threads across one partial
   constexpr int NG = 256 / LANES;         // groups of splits
   constexpr int PER = (64 + NG - 1) / NG; // splits a thread may own
@@ -1710,6 +1727,7 @@ __global__ void __launch_bounds__(256) attn_merge_kernel(const float* __restrict
     const float w_s = l_s > 0.f ? exp2f(m_s - big) : 0.f;
     float denom = 0.f;                     // in split order
     for (int s = 0; s < splits; ++s) denom += __shfl(w_s * l_s, s, WAVE);
+    if (sink != nullptr && big != -INFINITY) denom += exp2f(sink[h] * 1.4426950408889634f - big);
     weight[tid] = w_s;
     if (tid == 0) inv_denom = denom > 0.f ? 1.0f / denom : 0.f;
   }
@@ -1776,11 +1794,10 @@ extern "C" int holon_attention_mfma_supported(int head_dim, int page_size, int d
   return dtype == HOLON_BF16 && mfma_serves(head_dim, page_size);
 }
 
-extern "C" int holon_attention_prefill_bf16(const void* q, void* out, const void* pages, const int32_t* table,
-                                            int table_stride, const int32_t* slots, const int32_t* lens,
-                                            const int32_t* query_start, const int32_t* row_ids, int n_rows,
-                                            int max_query, int max_len, int heads, int kv_heads, int head_dim,
-                                            int page_size, float scale, int window, void* stream) {
+static int prefill_launch(const void* q, void* out, const void* pages, const int32_t* table, int table_stride,
+                          const int32_t* slots, const int32_t* lens, const int32_t* query_start, const int32_t* row_ids,
+                          int n_rows, int max_query, int max_len, int heads, int kv_heads, int head_dim, int page_size,
+                          float scale, int window, const float* sink, void* stream) {
   HOLON_CHECK(mfma_serves(head_dim, page_size), "attention (matrix cores): head_dim %d / page %d not served", head_dim,
               page_size);
   HOLON_CHECK(heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && window >= 0 && table_stride > 0,
@@ -1790,7 +1807,7 @@ extern "C" int holon_attention_prefill_bf16(const void* q, void* out, const void
   a.q = (const bf16_t*)q; a.out = (bf16_t*)out; a.pages = (const bf16_t*)pages; a.table = table;
   a.table_stride = table_stride; a.slots = slots; a.lens = lens; a.qstart = query_start; a.row_ids = row_ids;
   a.heads = heads; a.kv_heads = kv_heads; a.page_size = page_size;
-  a.scale_log2 = scale * 1.4426950408889634f; a.window = window;
+  a.scale_log2 = scale * 1.4426950408889634f; a.window = window; a.sink = sink;
   const TileMap tm = tile_map(heads / kv_heads);
   const int nt = head_dim == 256 ? 1 : 2;
   const int tiles = (max_query + tm.pos_per_tile - 1) / tm.pos_per_tile;
@@ -1843,6 +1860,26 @@ extern "C" int holon_attention_prefill_bf16(const void* q, void* out, const void
   else attn_prefill_kernel<256, 1><<<grid, 256, 0, s>>>(a);
   HOLON_LAUNCH_OK();
   return 0;
+}
+
+extern "C" int holon_attention_prefill_bf16(const void* q, void* out, const void* pages, const int32_t* table,
+                                            int table_stride, const int32_t* slots, const int32_t* lens,
+                                            const int32_t* query_start, const int32_t* row_ids, int n_rows,
+                                            int max_query, int max_len, int heads, int kv_heads, int head_dim,
+                                            int page_size, float scale, int window, void* stream) {
+  return prefill_launch(q, out, pages, table, table_stride, slots, lens, query_start, row_ids, n_rows, max_query, max_len,
+                        heads, kv_heads, head_dim, page_size, scale, window, nullptr, stream);
+}
+
+// The same with a sink per query head in the softmax's denominator (`sink` [heads] float32; null: none).
+extern "C" int holon_attention_prefill_sink_bf16(const void* q, void* out, const void* pages, const int32_t* table,
+                                                 int table_stride, const int32_t* slots, const int32_t* lens,
+                                                 const int32_t* query_start, const int32_t* row_ids, int n_rows,
+                                                 int max_query, int max_len, int heads, int kv_heads, int head_dim,
+                                                 int page_size, float scale, int window, const float* sink,
+                                                 void* stream) {
+  return prefill_launch(q, out, pages, table, table_stride, slots, lens, query_start, row_ids, n_rows, max_query, max_len,
+                        heads, kv_heads, head_dim, page_size, scale, window, sink, stream);
 }
 
 // Prompt portions of windowed attention with sigmoid weights (head sizes 64 and 128, keys and values of one width,
@@ -1912,7 +1949,8 @@ static int decode_launch(const void* q, void* out, const void* pages, const int3
                          const int32_t* slots, const int32_t* lens, const int32_t* query_start, const int32_t* row_ids,
                          int n_rows, int max_len, int heads, int kv_heads, int head_dim, int page_size, float scale,
                          int window, float* part_o, float* part_ml, int splits, int keys_per_split, void* stream,
-                         const FusedArgs* fused = nullptr, int waves = 1, int rows_in_order = 0) {
+                         const FusedArgs* fused = nullptr, int waves = 1, int rows_in_order = 0,
+                         const float* sink = nullptr) {
   HOLON_CHECK(mfma_serves(head_dim, page_size), "attention (matrix cores): head_dim %d / page %d not served", head_dim,
               page_size);
   HOLON_CHECK(heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && window >= 0 && table_stride > 0,
@@ -1924,7 +1962,8 @@ static int decode_launch(const void* q, void* out, const void* pages, const int3
               "partials within 64 KB of LDS)", waves, splits, head_dim);
   HOLON_CHECK(splits == waves || (part_o && part_ml), "attention decode: %d splits over blocks need a workspace",
               splits / waves);
-  const int span = window > 0 ? (window < max_len ? window + 31 : max_len) : max_len;
+  // (a window's keys are walked from a 32-key border on, and never more keys than the longest row holds)
+  const int span = window > 0 && window + 31 < max_len ? window + 31 : max_len;
   HOLON_CHECK((int64_t)splits * keys_per_split >= span, "attention decode: %d splits of %d keys do not cover %d keys",
               splits, keys_per_split, span);
   if (n_rows <= 0) return 0;
@@ -1934,7 +1973,7 @@ static int decode_launch(const void* q, void* out, const void* pages, const int3
   a.heads = heads; a.kv_heads = kv_heads; a.page_size = page_size;
   a.scale_log2 = scale * 1.4426950408889634f; a.window = window;
   a.part_o = part_o; a.part_ml = part_ml; a.splits = splits; a.keys_per_split = keys_per_split;
-  a.out_splits = splits / waves; a.rows_in_order = rows_in_order;
+  a.out_splits = splits / waves; a.rows_in_order = rows_in_order; a.sink = sink;
   const TileMap tm = tile_map(heads / kv_heads);
   dim3 grid(a.out_splits, kv_heads * tm.head_blocks, n_rows);
   hipStream_t s = (hipStream_t)stream;
@@ -1955,11 +1994,11 @@ static int decode_launch(const void* q, void* out, const void* pages, const int3
   splits = a.out_splits;
   dim3 mgrid(n_rows, heads);
   if (head_dim == 64)
-    attn_merge_kernel<64><<<mgrid, 256, 0, s>>>(part_o, part_ml, (bf16_t*)out, row_ids, query_start, heads, splits);
+    attn_merge_kernel<64><<<mgrid, 256, 0, s>>>(part_o, part_ml, (bf16_t*)out, row_ids, query_start, heads, splits, sink);
   else if (head_dim == 128)
-    attn_merge_kernel<128><<<mgrid, 256, 0, s>>>(part_o, part_ml, (bf16_t*)out, row_ids, query_start, heads, splits);
+    attn_merge_kernel<128><<<mgrid, 256, 0, s>>>(part_o, part_ml, (bf16_t*)out, row_ids, query_start, heads, splits, sink);
   else
-    attn_merge_kernel<256><<<mgrid, 256, 0, s>>>(part_o, part_ml, (bf16_t*)out, row_ids, query_start, heads, splits);
+    attn_merge_kernel<256><<<mgrid, 256, 0, s>>>(part_o, part_ml, (bf16_t*)out, row_ids, query_start, heads, splits, sink);
   HOLON_LAUNCH_OK();
   return 0;
 }
@@ -1987,6 +2026,19 @@ extern "C" int holon_attention_decode_waves_bf16(const void* q, void* out, const
   return decode_launch(q, out, pages, table, table_stride, slots, lens, query_start, row_ids, n_rows, max_len, heads,
                        kv_heads, head_dim, page_size, scale, window, part_o, part_ml, splits, keys_per_split, stream,
                        nullptr, waves, rows_in_order);
+}
+
+// The same with a sink per query head in the softmax's denominator (`sink` [heads] float32; null: none).
+extern "C" int holon_attention_decode_sink_bf16(const void* q, void* out, const void* pages, const int32_t* table,
+                                                int table_stride, const int32_t* slots, const int32_t* lens,
+                                                const int32_t* query_start, const int32_t* row_ids, int n_rows,
+                                                int max_len, int heads, int kv_heads, int head_dim, int page_size,
+                                                float scale, int window, float* part_o, float* part_ml, int splits,
+                                                int keys_per_split, int waves, int rows_in_order, const float* sink,
+                                                void* stream) {
+  return decode_launch(q, out, pages, table, table_stride, slots, lens, query_start, row_ids, n_rows, max_len, heads,
+                       kv_heads, head_dim, page_size, scale, window, part_o, part_ml, splits, keys_per_split, stream,
+                       nullptr, waves, rows_in_order, sink);
 }
 
 // Decode rows straight from the step's raw q/k/v projection: per-head norm, rotation and the cache write of each

@@ -69,6 +69,19 @@ int holon_attention_decode_waves_bf16(const void* q, void* out, const void* page
                                       int heads, int kv_heads, int head_dim, int page_size, float scale, int window,
                                       float* part_o, float* part_ml, int splits, int keys_per_split, int waves,
                                       int rows_in_order, void* stream);
+// The prompt and the decode entry points with a sink per query head in the softmax's denominator (`sink` [heads]
+// float32 in the scores' units, or NULL): exp(sink - max) is added to the sum of the weights; it has no key or value.
+int holon_attention_prefill_sink_bf16(const void* q, void* out, const void* pages, const int32_t* table,
+                                      int table_stride, const int32_t* slots, const int32_t* lens,
+                                      const int32_t* query_start, const int32_t* row_ids, int n_rows, int max_query,
+                                      int max_len, int heads, int kv_heads, int head_dim, int page_size, float scale,
+                                      int window, const float* sink, void* stream);
+int holon_attention_decode_sink_bf16(const void* q, void* out, const void* pages, const int32_t* table,
+                                     int table_stride, const int32_t* slots, const int32_t* lens,
+                                     const int32_t* query_start, const int32_t* row_ids, int n_rows, int max_len,
+                                     int heads, int kv_heads, int head_dim, int page_size, float scale, int window,
+                                     float* part_o, float* part_ml, int splits, int keys_per_split, int waves,
+                                     int rows_in_order, const float* sink, void* stream);
 // The same from the step's raw q/k/v projection `qkv` [T, (heads + 2 kv_heads) head_dim]: per-head RMSNorm (q_weight
 // and k_weight, both or neither), rotation (rope_table [max_positions, head_dim] = cos | sin, or NULL) and the cache
 // write of every row's new token (write_page, write_off by token; its position is the row's len - 1) happen inside

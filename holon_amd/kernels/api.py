@@ -133,10 +133,16 @@ class Kernels(Protocol):
         """Raise, with a message that names the limit, when no attention kernel serves this head size, page size and
         dtype. Mixers call it when they are built, so that a model is refused before it takes a request."""
 
+    def attention_on_cores(self, head_dim: int, page_size: int, dtype: torch.dtype) -> bool:
+        """Whether `paged_attention` runs on the matrix cores at this head size, page size and dtype (there it also
+        takes a sink)."""
+        return False
+
     def paged_attention(self, q: torch.Tensor, pages: torch.Tensor, table: torch.Tensor, rows: AttnRows,
-                        page_size: int, scale: float, window: int) -> torch.Tensor:
+                        page_size: int, scale: float, window: int, sink: torch.Tensor | None = None) -> torch.Tensor:
         """softmax(q k^T * scale) v per row over its cached tokens, causal; with window W > 0 a query at position p
-        sees keys p-W+1 .. p. q [T, Hq, D] -> [T, Hq, D]. This step's keys are already in the cache."""
+        sees keys p-W+1 .. p. q [T, Hq, D] -> [T, Hq, D]. This step's keys are already in the cache. `sink` [Hq]
+        float32: exp(sink[h] - max) is added to the softmax's denominator (it has no key and no value)."""
 
     def qkv_attention(self, qkv: torch.Tensor, heads: int, kv_heads: int, head_dim: int,
                       q_weight: torch.Tensor | None, k_weight: torch.Tensor | None, eps: float,

@@ -74,6 +74,10 @@ class HipKernels:
             "holon_attention_prefill_copies": [_I],
             "holon_attention_decode_waves_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I,
                                                   _P, _P, _I, _I, _I, _I, _P],
+            "holon_attention_prefill_sink_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I,
+                                                  _P, _P],
+            "holon_attention_decode_sink_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I,
+                                                 _P, _P, _I, _I, _I, _I, _P, _P],
             "holon_attention_decode_fused_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I,
                                                   _P, _P, _F, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _P],
             "holon_gemm_skinny_supported": [_I, _I, _I],
@@ -631,7 +635,10 @@ class HipKernels:
             raise KernelError(f"attention: head_dim {head_dim} is not served (multiples of 8 up to 512, any page size "
                               f">= 1; got page size {page_size})")
 
-    def paged_attention(self, q, pages, table, rows: AttnRows, page_size, scale, window):
+    def attention_on_cores(self, head_dim, page_size, dtype) -> bool:
+        return bool(dtype in _DT and self.lib.holon_attention_mfma_supported(head_dim, page_size, _DT[dtype]))
+
+    def paged_attention(self, q, pages, table, rows: AttnRows, page_size, scale, window, sink=None):
         self._check(q, "attention q")
         self._check(pages, "attention pages", q.dtype)
         self._check(table, "block table", torch.int32)
@@ -641,22 +648,29 @@ class HipKernels:
             raise KernelError(f"attention: pages {tuple(pages.shape)} do not fit head_dim {d}, page {page_size}")
         out = torch.empty_like(q)
         b = rows.slots.shape[0]
+        if sink is not None:
+            self._check(sink, "attention sink", torch.float32)
+            if sink.shape != (hq,):
+                raise KernelError(f"attention: sink {tuple(sink.shape)} for {hq} heads")
         if self.lib.holon_attention_mfma_supported(d, page_size, self._dt(q, "attention")):
             common = (q.data_ptr(), out.data_ptr(), pages.data_ptr(), table.data_ptr(), table.shape[1],
                       rows.slots.data_ptr(), rows.lens.data_ptr(), rows.query_start.data_ptr())
             if rows.n_chunk:
-                self._call(self.lib.holon_attention_prefill_bf16, *common, rows.chunk_rows.data_ptr(), rows.n_chunk,
+                self._call(self.lib.holon_attention_prefill_sink_bf16, *common, rows.chunk_rows.data_ptr(), rows.n_chunk,
                            rows.max_chunk_query, rows.max_chunk_len, hq, hkv, d, page_size, float(scale), int(window),
-                           self._stream())
+                           _ptr(sink), self._stream())
             if rows.n_decode:
                 span = rows.max_decode_len if not window else min(rows.max_decode_len, window + 31)
                 splits, per, waves = self.decode_splits(rows.n_decode * hkv * ((hq // hkv + 15) // 16), span, d)
                 part_o, part_ml = self._decode_parts(rows.n_decode * hq * (splits // waves), d, q.device)
-                self._call(self.lib.holon_attention_decode_waves_bf16, *common, rows.decode_rows.data_ptr(),
+                self._call(self.lib.holon_attention_decode_sink_bf16, *common, rows.decode_rows.data_ptr(),
                            rows.n_decode, rows.max_decode_len, hq, hkv, d, page_size, float(scale), int(window),
                            _ptr(part_o), _ptr(part_ml), splits, per, waves, int(rows.in_order and rows.n_decode == t),
-                           self._stream())
+                           _ptr(sink), self._stream())
             return out
+        if sink is not None:
+            raise KernelError("attention: a sink is served by the matrix-core kernels (and by `softmax_attention`), "
+                              f"not at head_dim {d}, page {page_size}, {q.dtype}")
         self._call(self.lib.holon_attention_generic, q.data_ptr(), out.data_ptr(), pages.data_ptr(), table.data_ptr(),
                    table.shape[1], rows.slots.data_ptr(), rows.lens.data_ptr(), rows.query_start.data_ptr(), b, t, hq,
                    hkv, d, page_size, pages.shape[0], float(scale), int(window), self._dt(q, "attention"),

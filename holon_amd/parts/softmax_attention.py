@@ -89,6 +89,17 @@ register_kernel(KernelOp("softmax_attention", softmax_attention_plain, "holon_so
 register_kernel(KernelOp("head_linear", head_linear_plain))
 
 
+def attend(k, q, held, view, step, kv_heads, vdim, sink, scale, window):
+    """The attention of both mixers: on the matrix cores where keys and values have one width that those kernels
+    serve (the pages' layout is then theirs), else the general kernel. q [T, H, D] -> [T, H V]."""
+    t, heads, dim = q.shape
+    if dim == vdim and k.attention_on_cores(dim, view.page_size, q.dtype):
+        pages = held.pages.view(-1, 2, kv_heads, view.page_size * dim)
+        return k.paged_attention(q, pages, view.table, step.rows, view.page_size, scale, window, sink=sink).view(t, heads * vdim)
+    return k.softmax_attention(q, held.pages, view.table, step.rows, step.token_row, step.positions, kv_heads, vdim,
+                               view.page_size, sink, scale, window)
+
+
 def to_half_split(rows_per_head: int, heads: int, rot: int) -> torch.Tensor:
     """The order of a projection's output rows that turns the interleaved pairing of rotary dimensions, (2i, 2i + 1),
     into the half-split one, (i, i + rot/2), head by head; rows from `rot` on stay. Queries and keys permuted alike
@@ -162,9 +173,8 @@ class SoftmaxAttention(Part):
         table = getattr(self.position, "table", None)
         q = k.head_prepare(self.qkv(x), self.heads, self.kv_heads, self.dim, self.vdim, None, None, 0.0, table,
                            step.positions, held.pages, view.write_page, view.write_off, view.page_size, bias=self.bias)
-        out = k.softmax_attention(q, held.pages, view.table, step.rows, step.token_row, step.positions, self.kv_heads,
-                                  self.vdim, view.page_size, self.sink if self.has_sink else None, self.scale,
-                                  self.window)
+        out = attend(k, q, held, view, step, self.kv_heads, self.vdim, self.sink if self.has_sink else None, self.scale,
+                     self.window)
         return self.o(out)
 
     __call__ = forward
@@ -229,8 +239,7 @@ class LatentAttention(Part):
         k.kv_write(c, c, held.pages.view(-1, 2, 1, view.page_size * self.kv_rank), view.write_page, view.write_off,
                    view.page_size)
         q = k.head_linear(self.uq(cq).view(t, self.heads, self.dim), self.uk_t)
-        mixed = k.softmax_attention(q, held.pages, view.table, step.rows, step.token_row, step.positions, 1,
-                                    self.kv_rank, view.page_size, None, self.scale, self.window)
+        mixed = attend(k, q, held, view, step, 1, self.kv_rank, None, self.scale, self.window)
         out = k.head_linear(mixed.view(t, self.heads, self.kv_rank), self.uv_h)
         return self.o(out.view(t, self.heads * self.vdim))
 

@@ -31,7 +31,9 @@ SHORT = (("_Z18gemm_skinny_kernelILi", "gemm_skinny<"), ("_Z22gemm_skinny_glu_ke
          ("_ZN12_GLOBAL__N_119head_prepare_kernelI", "head_prepare<"), ("_ZN12_GLOBAL__N_120delta_prepare_kernelI", "delta_prepare<"),
          ("_ZN12_GLOBAL__N_116gated_out_kernelI", "gated_out<"), ("_ZN12_GLOBAL__N_116shift_mix_kernelI", "shift_mix<"),
          ("_ZN12_GLOBAL__N_117shift_keep_kernelI", "shift_keep<"), ("_ZN12_GLOBAL__N_117decay_lora_kernelI", "decay_lora<"),
-         ("_ZN12_GLOBAL__N_120memory_pieces_kernel", "memory_pieces"), ("Cijk_Alik_Bljk_BBS_BH_Bias_HA_S_SAV_UserArgs_", "hipBLASLt "),
+         ("_ZN12_GLOBAL__N_120memory_pieces_kernel", "memory_pieces"),
+         ("_ZN12_GLOBAL__N_124softmax_attention_kernelI", "softmax_attention<"),
+         ("_ZN12_GLOBAL__N_117mlstm_scan_kernelILi", "mlstm_scan<"), ("_ZN12_GLOBAL__N_117dyt_stream_kernelI", "dyt_stream<"), ("Cijk_Alik_Bljk_BBS_BH_Bias_HA_S_SAV_UserArgs_", "hipBLASLt "),
          ("Custom_Cijk_Alik_Bljk_BBS_BH_Bias_HA_S_SAV_NTD_SK3_UserArgs_", "hipBLASLt custom "))
 
 
@@ -52,10 +54,10 @@ def dispatches(path: str) -> list[tuple]:
     return [(n, st, en, gx // max(wx, 1), gy, gz) for n, st, en, gx, gy, gz, wx in rows]
 
 
-CLASSES = (("attention", ("attn_", "sigmoid_attention")), ("matrix products", ("gemm_", "Cijk_", "Custom_Cijk_", "hipBLASLt")),
-           ("recurrent scans", ("memory_scan", "delta_scan", "memory_pieces", "delta_pieces")),
+CLASSES = (("attention", ("attn_", "sigmoid_attention", "softmax_attention")), ("matrix products", ("gemm_", "Cijk_", "Custom_Cijk_", "hipBLASLt")),
+           ("recurrent scans", ("memory_scan", "delta_scan", "memory_pieces", "delta_pieces", "mlstm_scan")),
            ("elementwise", ("rmsnorm", "silu_mul", "qk_norm_rope", "v_write", "kv_write", "embedding", "sum_parts",
-                            "row_sumsq", "scatter_rows", "stream_norm", "widen_", "pair_rows", "softcap", "causal_conv",
+                            "row_sumsq", "scatter_rows", "stream_norm", "dyt_stream", "widen_", "pair_rows", "softcap", "causal_conv",
                             "head_prepare", "delta_prepare", "gated_out", "shift_mix", "shift_keep", "decay_lora")),
            ("sampling", ("argmax", "sample_kernel", "store_tokens", "logprobs")))
 

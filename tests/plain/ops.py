@@ -164,7 +164,13 @@ class TorchKernels:
     def check_attention(self, head_dim, page_size, dtype):
         return None
 
-    def paged_attention(self, q, pages, table, rows, page_size, scale, window):
+    cores = False            # a test may switch it on: mixers then take the path they take where the matrix-core
+                             # attention kernels serve their sizes
+
+    def attention_on_cores(self, head_dim, page_size, dtype):
+        return self.cores
+
+    def paged_attention(self, q, pages, table, rows, page_size, scale, window, sink=None):
         t, hq, d = q.shape
         hkv = pages.shape[2]
         kp = pages[:, 0].view(-1, hkv, page_size, d)
@@ -184,7 +190,10 @@ class TorchKernels:
             hidden = key > pos
             if window:
                 hidden = hidden | (pos - key >= window)
-            probs = scores.masked_fill(hidden, float("-inf")).softmax(-1)
+            scores = scores.masked_fill(hidden, float("-inf"))
+            if sink is not None:             # a column of its own in the softmax, dropped again: it has no value
+                scores = torch.cat((scores, _up(sink)[:, None, None].expand(hq, e - s, 1)), dim=-1)
+            probs = scores.softmax(-1)[..., :n]
             out[s:e] = torch.einsum("hqk,khd->qhd", probs, v).to(q.dtype)
         return out
 

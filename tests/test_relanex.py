@@ -126,6 +126,21 @@ def test_float32_does_not_depend_on_the_cut(folders, device):
             assert H.rel_rms(row, whole[key]) < 1e-5, f"{key}: logits depend on how the prompt was cut"
 
 
+def test_the_matrix_core_path_of_the_mixers_on_the_twin(folders):
+    """Where keys and values have one width that the matrix-core attention kernels serve, both attention mixers hand
+    their pages to `paged_attention` (with the sink); the twin is told to say it serves them, and the logits stay the
+    plain model's."""
+    folder, requests = folders["D-sharp"], _requests("D-sharp", (40, 33, 21))
+    from holon_amd.engine.loading import load_model
+    from holon_amd.engine.replay import Replayer
+    kernels = TorchKernels()
+    kernels.cores = True
+    rep = Replayer(load_model(folder, device="cpu", dtype="float32", kernels=kernels, page_size=16, max_seqs=3,
+                              max_model_len=128, max_step_tokens=128, cache_tokens=128))
+    got = H.run_trace(rep, H.trace_mixed(requests, seed=2, max_live=3, decode_tail=5))
+    _check(folder, "float32", requests, got, "matrix-core path on the twin")
+
+
 def _needle_model(root, window, page):
     """One latent-attention layer (no positions: a score depends on the two tokens alone). A pair of token ids (query
     token, key token) whose score is the largest of all, and a filler token whose scores with them and with itself
@@ -403,6 +418,42 @@ def test_kernels_against_their_plain_forms(dtype):
         gate, wn = proj[:, 2 * hd + hv: 2 * hd + 2 * hv], rn(hv).to(dtype)
         assert _rel(k.gated_out(o1, gate, wn, True, 1e-6, dtype, act="sigmoid"),
                     kernel_op("gated_out").plain(o1, gate, wn, True, 1e-6, dtype, act="sigmoid")) < tol
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("d,heads,kv,window", [(64, 8, 2, 0), (128, 16, 4, 100), (128, 8, 8, 0), (256, 16, 1, 333),
+                                               (64, 40, 1, 0)])
+def test_the_sink_on_the_matrix_cores(d, heads, kv, window):
+    """`paged_attention` with a sink in bfloat16 at the head sizes the matrix-core kernels serve: long and short
+    prompt portions and decode rows of several lengths in one step, against the plain form."""
+    from holon_amd.kernels import load_hip
+    from holon_amd.kernels.api import AttnRows
+    k, dev, page = load_hip(), "cuda", 16
+    g = torch.Generator(device=dev).manual_seed(d + heads)
+    rn = lambda *s: torch.randn(*s, device=dev, generator=g)      # noqa: E731
+    lens, nq = [700, 40, 900, 33, 1], [300, 5, 1, 1, 1]
+    most = -(-max(lens) // page)
+    n_rows = len(lens)
+    pages = rn(n_rows * most + 1, 2, kv, page * d).bfloat16()
+    table = torch.full((n_rows + 1, most), n_rows * most, dtype=torch.int32)
+    table[:n_rows] = torch.randperm(n_rows * most).view(n_rows, most).int()
+    table = table.to(dev)
+    qs = [0]
+    for n in nq:
+        qs.append(qs[-1] + n)
+    as_i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)      # noqa: E731
+    rows = AttnRows(slots=as_i32(list(range(n_rows))), lens=as_i32(lens), query_start=as_i32(qs),
+                    decode_rows=as_i32([2, 3, 4]), chunk_rows=as_i32([0, 1]), n_decode=3, n_chunk=2, max_decode_len=900,
+                    max_chunk_query=300, max_chunk_len=700)
+    q = rn(sum(nq), heads, d).bfloat16()
+    scale = 2.0 * d ** -0.5
+    sink = 2.0 * rn(heads) + 2.0
+    for with_sink in (sink, None):
+        got = k.paged_attention(q, pages, table, rows, page, scale, window, sink=with_sink)
+        want = TorchKernels().paged_attention(q.float(), pages.float(), table, rows, page, scale, window, sink=with_sink)
+        assert H.rel_rms(got.float(), want) < 1e-2, (d, heads, kv, window, with_sink is not None)
+    assert H.rel_rms(k.paged_attention(q, pages, table, rows, page, scale, window, sink=sink).float(),
+                     k.paged_attention(q, pages, table, rows, page, scale, window).float()) > 0.05      # the sink shows
 
 
 @pytest.mark.gpu
