@@ -275,11 +275,14 @@ int holon_softmax_attention(const void* q, void* out, const void* pages, const i
 // -- the matrix memory of xLSTM (mlstm.hip) -------------------------------------------------------------------------------
 // proj [T, width]: q, k [H D] and v [H V] and the gates' pre-activations [2 H] (input, then forget) from the given
 // columns; gate_bias [2 H]; state S [slots, H, D, V], n [slots, H, ceil(V / 8), D], m [slots, H, ceil(V / 8)] (a copy
-// for every 8 value columns), float32; out [T, H, V] float32.
+// for every 8 value columns), float32; out [T, H, V] float32. piece_tokens > 0: rows are cut into pieces of that many
+// tokens that run side by side in two passes (at most max_pieces a row; piece_base [rows]: the number of each row's
+// first piece among all; workspaces gates [T, H, 3], sloc [pieces, H, D, V], nloc [pieces, H, D], pk [pieces, H]).
 int holon_mlstm_scan(const void* proj, int width, int q_off, int k_off, int v_off, int gate_off, const float* gate_bias,
                      float cap, float* S, float* n, float* m, float* out, const int32_t* slots, const int32_t* starts,
                      const int32_t* query_start, int rows, int heads, int dim, int vdim, int state_slots, int dtype,
-                     void* stream);
+                     int tokens, int piece_tokens, int max_pieces, const int32_t* piece_base, float* gates, float* sloc,
+                     float* nloc, float* pk, void* stream);
 
 #ifdef __cplusplus
 }

@@ -13,6 +13,13 @@
 // the batch before is worked through; the gates' functions are taken then, off the recurrence's path.
 // The blocks of a head (one for every 8 columns) all need n and m and do not wait for each other, so each keeps a copy
 // of its own in the slot, n [H, V/8, D] and m [H, V/8]: a block reads and writes nothing that another block touches.
+//
+// Long rows run in pieces side by side. The maxima depend on the gates alone, m' = max(m + f, i), a recurrence whose
+// steps compose ((a, b) then (c, d) is (a + c, max(b + c, d))), so a wave finds a whole row's maxima by a prefix scan and
+// leaves every token's two factors exp(f + m - m') and exp(i - m') and exp(-m') behind. With those the recurrence is
+// linear in S and n with factors that do not depend on them: every piece but a row's last first runs from zero and
+// leaves what it adds and the product of its factors; a small kernel walks a row's pieces in order, leaving each
+// piece's true start; then every piece runs again from there and writes its outputs.
 #include "common.h"
 #include "holon_hip.h"
 
@@ -35,6 +42,96 @@ __device__ __forceinline__ float log_sigmoid(float x) {   // -softplus(-x), with
   return fminf(x, 0.f) - log1pf(expf(-fabsf(x)));
 }
 
+struct MlstmPieces {
+  int tokens;                  // tokens a piece (0: rows are not cut, the gates are taken inside the scan)
+  int mode;                    // 1: from zero, leave what the piece adds; 2: from the true start, write outputs
+  const int32_t* base;         // [rows]: the number of row b's first piece among all pieces of the step
+  const float* gates;          // [T, H, 3]: exp(f + m - m'), exp(i - m'), exp(-m') of every token
+  float* sloc;                 // [pieces, H, D, V]
+  float* nloc;                 // [pieces, H, D]
+  float* pk;                   // [pieces, H]
+};
+
+// One wave per (row, head): the row's maxima by a prefix scan over lanes that each hold a run of neighbouring tokens,
+// then every token's three factors. The slot's copies of m take the row's last maximum.
+template <typename T>
+__global__ void __launch_bounds__(WAVE) mlstm_gates_kernel(const T* __restrict__ proj, int width, int gate_off,
+                                                           const float* __restrict__ gate_bias, float cap,
+                                                           float* __restrict__ m_all, float* __restrict__ gates,
+                                                           const int32_t* __restrict__ slots,
+                                                           const int32_t* __restrict__ starts,
+                                                           const int32_t* __restrict__ query_start, int heads,
+                                                           int copies) {
+  const int b = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int lo = query_start[b], hi = query_start[b + 1], n = hi - lo;
+  if (n <= 0) return;
+  const int64_t cell = ((int64_t)slots[b] * heads + h) * copies;
+  const float m0 = starts[b] > 0 ? m_all[cell] : 0.f;
+  const float bi = gate_bias[h], bf = gate_bias[heads + h];
+  const int seg = (n + WAVE - 1) / WAVE;
+  const int t0 = lo + lane * seg, t1 = min(hi, t0 + seg);
+  auto gate = [&](int t, float& it, float& ft) {
+    const T* row = proj + (int64_t)t * width + gate_off;
+    it = cap * tanhf((Elem<T>::load(row[h]) + bi) / cap);
+    ft = log_sigmoid(cap * tanhf((Elem<T>::load(row[heads + h]) + bf) / cap));
+  };
+  float A = 0.f, B = -INFINITY;                       // this lane's run as one step: m -> max(m + A, B)
+  for (int t = t0; t < t1; ++t) {
+    float it, ft;
+    gate(t, it, ft);
+    B = fmaxf(B + ft, it);
+    A += ft;
+  }
+#pragma unroll
+  for (int off = 1; off < WAVE; off <<= 1) {           // inclusive scan: the runs of lanes 0 .. lane as one step
+    const float Ao = __shfl_up(A, off, WAVE), Bo = __shfl_up(B, off, WAVE);
+    if (lane >= off) {
+      B = fmaxf(Bo + A, B);
+      A = Ao + A;
+    }
+  }
+  const float Ae = __shfl_up(A, 1, WAVE), Be = __shfl_up(B, 1, WAVE);
+  float m = lane == 0 ? m0 : fmaxf(m0 + Ae, Be);
+  for (int t = t0; t < t1; ++t) {
+    float it, ft;
+    gate(t, it, ft);
+    const float m_new = fmaxf(ft + m, it);
+    float* g = gates + ((int64_t)t * heads + h) * 3;
+    g[0] = expf(ft + m - m_new);
+    g[1] = expf(it - m_new);
+    g[2] = expf(-m_new);
+    m = m_new;
+  }
+  if (t0 < hi && t1 == hi)
+    for (int c = 0; c < copies; ++c) m_all[cell + c] = m;
+}
+
+// A row's pieces in order: S <- pk S + sloc (n likewise); sloc[p] becomes the state piece p + 1 starts from.
+__global__ void __launch_bounds__(256) mlstm_pieces_kernel(const float* __restrict__ S_all, const float* __restrict__ n_all,
+                                                           const int32_t* __restrict__ slots,
+                                                           const int32_t* __restrict__ starts,
+                                                           const int32_t* __restrict__ query_start, int heads, int dim,
+                                                           int vdim, int copies, MlstmPieces pc) {
+  const int b = blockIdx.x, h = blockIdx.y;
+  const int n = query_start[b + 1] - query_start[b];
+  const int pieces = (n + pc.tokens - 1) / pc.tokens;
+  if (pieces < 2) return;
+  const int64_t cell = (int64_t)slots[b] * heads + h;
+  const bool carried = starts[b] > 0;
+  const int64_t first = pc.base[b];
+  const int cells = dim * vdim;
+  for (int e = threadIdx.x; e < cells + dim; e += 256) {
+    const bool of_n = e >= cells;
+    float x = !carried ? 0.f : of_n ? n_all[cell * copies * dim + (e - cells)] : S_all[cell * cells + e];
+    for (int p = 0; p < pieces - 1; ++p) {
+      const int64_t at = (first + p) * heads + h;
+      float* add = of_n ? pc.nloc + at * dim + (e - cells) : pc.sloc + at * cells + e;
+      x = pc.pk[at] * x + *add;
+      *add = x;
+    }
+  }
+}
+
 template <int KD, typename T>
 __global__ void __launch_bounds__(WAVE) mlstm_scan_kernel(const T* __restrict__ proj, int width, int q_off, int k_off,
                                                           int v_off, int gate_off, const float* __restrict__ gate_bias,
@@ -43,16 +140,30 @@ __global__ void __launch_bounds__(WAVE) mlstm_scan_kernel(const T* __restrict__ 
                                                           const int32_t* __restrict__ slots,
                                                           const int32_t* __restrict__ starts,
                                                           const int32_t* __restrict__ query_start, int heads, int dim,
-                                                          int vdim) {
+                                                          int vdim, int col_blocks, MlstmPieces pc) {
   constexpr int KQ = KD / PARTS, TC = KD <= 64 ? 16 : KD <= 128 ? 8 : 4, N = TC * KD, PER = (N + WAVE - 1) / WAVE;
   __shared__ float qs[2][N], ks[2][N];
-  __shared__ float vs[2][TC * COLS], gi[2][TC], gf[2][TC];
-  const int b = blockIdx.x, h = blockIdx.y, col_block = blockIdx.z, lane = threadIdx.x;
+  __shared__ float vs[2][TC * COLS], gi[2][TC], gf[2][TC], ge[2][TC];
+  const int b = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int piece = blockIdx.z / col_blocks, col_block = blockIdx.z % col_blocks;
   const int part = lane % PARTS, col = lane / PARTS, j = col_block * COLS + col;
   const bool active = j < vdim;
-  const int lo = query_start[b], hi = query_start[b + 1];
+  int lo = query_start[b], hi = query_start[b + 1];
+  const bool cut = pc.tokens > 0;                      // (the gates then come as factors: gi = keep, gf = take, ge = exp(-m))
+  bool from_slot = true, to_slot = true;
+  int64_t piece_no = 0;
+  if (cut) {                                           // (everything here is the same in all of the block's lanes)
+    const int pieces = (hi - lo + pc.tokens - 1) / pc.tokens;
+    if (piece >= pieces || (pc.mode == 1 && piece == pieces - 1)) return;
+    lo += piece * pc.tokens;
+    hi = min(hi, lo + pc.tokens);
+    from_slot = piece == 0;
+    to_slot = pc.mode == 2 && piece == pieces - 1;
+    piece_no = pc.base[b] + piece;
+  }
+  const bool local = cut && pc.mode == 1;
   const int64_t cell = (int64_t)slots[b] * heads + h;
-  const int64_t mine = cell * gridDim.z + col_block;         // this block's own copy of n and m
+  const int64_t mine = cell * col_blocks + col_block;        // this block's own copy of n and m
   float* S_held = S_all + cell * dim * vdim;
   float* n_held = n_all + mine * dim;
   const bool carried = starts[b] > 0;
@@ -60,13 +171,22 @@ __global__ void __launch_bounds__(WAVE) mlstm_scan_kernel(const T* __restrict__ 
 #pragma unroll
   for (int i = 0; i < KQ; ++i) {
     const int row = part * KQ + i;
-    S[i] = (carried && active && row < dim) ? S_held[(int64_t)row * vdim + j] : 0.f;
-    nn[i] = (carried && row < dim) ? n_held[row] : 0.f;
+    if (local) {
+      S[i] = nn[i] = 0.f;
+    } else if (from_slot) {
+      S[i] = (carried && active && row < dim) ? S_held[(int64_t)row * vdim + j] : 0.f;
+      nn[i] = (carried && row < dim) ? n_held[row] : 0.f;
+    } else {
+      const int64_t at = (piece_no - 1) * heads + h;
+      S[i] = (active && row < dim) ? pc.sloc[at * dim * vdim + (int64_t)row * vdim + j] : 0.f;
+      nn[i] = row < dim ? pc.nloc[at * dim + row] : 0.f;
+    }
   }
-  float m = carried ? m_all[mine] : 0.f;
+  float m = (carried && !cut) ? m_all[mine] : 0.f;
+  float pk = 1.f;
   const float q_scale = 1.0f / sqrtf((float)dim);
   const float bi = gate_bias[h], bf = gate_bias[heads + h];
-  float nq[PER], nk[PER], ngi = 0.f, ngf = 0.f;
+  float nq[PER], nk[PER], ngi = 0.f, ngf = 0.f, nge = 0.f;
   auto ask = [&](int t0) {
 #pragma unroll
     for (int e = 0; e < PER; ++e) {
@@ -78,10 +198,17 @@ __global__ void __launch_bounds__(WAVE) mlstm_scan_kernel(const T* __restrict__ 
     }
     static_assert(TC * COLS <= 2 * WAVE, "a lane stages at most two values of v");
     if (lane < TC && t0 + lane < hi) {
-      const T* row = proj + (int64_t)(t0 + lane) * width;
-      const float ai = Elem<T>::load(row[gate_off + h]) + bi, af = Elem<T>::load(row[gate_off + heads + h]) + bf;
-      ngi = cap * tanhf(ai / cap);
-      ngf = log_sigmoid(cap * tanhf(af / cap));
+      if (cut) {
+        const float* g = pc.gates + ((int64_t)(t0 + lane) * heads + h) * 3;
+        ngi = g[0];
+        ngf = g[1];
+        nge = g[2];
+      } else {
+        const T* row = proj + (int64_t)(t0 + lane) * width;
+        const float ai = Elem<T>::load(row[gate_off + h]) + bi, af = Elem<T>::load(row[gate_off + heads + h]) + bf;
+        ngi = cap * tanhf(ai / cap);
+        ngf = log_sigmoid(cap * tanhf(af / cap));
+      }
     }
   };
   float nv2[2];
@@ -104,7 +231,7 @@ __global__ void __launch_bounds__(WAVE) mlstm_scan_kernel(const T* __restrict__ 
       const int idx = lane + e * WAVE;
       if (idx < TC * COLS) vs[buf][idx] = nv2[e];
     }
-    if (lane < TC) { gi[buf][lane] = ngi; gf[buf][lane] = ngf; }
+    if (lane < TC) { gi[buf][lane] = ngi; gf[buf][lane] = ngf; ge[buf][lane] = nge; }
   };
   if (lo < hi) {
     ask(lo);
@@ -119,13 +246,31 @@ __global__ void __launch_bounds__(WAVE) mlstm_scan_kernel(const T* __restrict__ 
     }
     const int nt = min(TC, hi - t0);
     for (int tt = 0; tt < nt; ++tt) {
-      const float it = gi[buf][tt], ft = gf[buf][tt];
-      const float m_new = fmaxf(ft + m, it);
-      const float keep = expf(ft + m - m_new), take = expf(it - m_new);
-      m = m_new;
+      float keep, take, floor_;
+      if (cut) {
+        keep = gi[buf][tt];
+        take = gf[buf][tt];
+        floor_ = ge[buf][tt];
+      } else {
+        const float it = gi[buf][tt], ft = gf[buf][tt];
+        const float m_new = fmaxf(ft + m, it);
+        keep = expf(ft + m - m_new);
+        take = expf(it - m_new);
+        m = m_new;
+        floor_ = expf(-m);
+      }
       const float vt = vs[buf][tt * COLS + col] * take;
       const float* qt = &qs[buf][tt * KD + part * KQ];
       const float* kt = &ks[buf][tt * KD + part * KQ];
+      if (local) {                       // what the piece adds, and the product of its factors; no output yet
+#pragma unroll
+        for (int i = 0; i < KQ; ++i) {
+          S[i] = keep * S[i] + kt[i] * vt;
+          nn[i] = keep * nn[i] + take * kt[i];
+        }
+        pk *= keep;
+        continue;
+      }
       float o = 0.f, d = 0.f;
 #pragma unroll
       for (int i = 0; i < KQ; ++i) {
@@ -136,13 +281,26 @@ __global__ void __launch_bounds__(WAVE) mlstm_scan_kernel(const T* __restrict__ 
       }
       o = part_sum(o);
       d = part_sum(d);
-      const float den = fmaxf(fabsf(d), expf(-m)) + 1e-6f;
+      const float den = fmaxf(fabsf(d), floor_) + 1e-6f;
       if (active && part == 0) out[((int64_t)(t0 + tt) * heads + h) * vdim + j] = o / den;
     }
     if (t0 + TC < hi) put(buf ^ 1);
     __syncthreads();
   }
   if (lo >= hi) return;
+  if (local) {
+    const int64_t at = piece_no * heads + h;
+#pragma unroll
+    for (int i = 0; i < KQ; ++i) {
+      const int row = part * KQ + i;
+      if (row >= dim) continue;
+      if (active) pc.sloc[at * dim * vdim + (int64_t)row * vdim + j] = S[i];
+      if (col_block == 0 && col == 0) pc.nloc[at * dim + row] = nn[i];
+    }
+    if (col_block == 0 && lane == 0) pc.pk[at] = pk;
+    return;
+  }
+  if (!to_slot) return;
 #pragma unroll
   for (int i = 0; i < KQ; ++i) {
     const int row = part * KQ + i;
@@ -150,15 +308,15 @@ __global__ void __launch_bounds__(WAVE) mlstm_scan_kernel(const T* __restrict__ 
     if (active) S_held[(int64_t)row * vdim + j] = S[i];
     if (col == 0) n_held[row] = nn[i];
   }
-  if (lane == 0) m_all[mine] = m;
+  if (lane == 0 && !cut) m_all[mine] = m;              // (cut: the gates' kernel has left the row's last maximum)
 }
 
 template <typename T, int KD>
 void launch_mlstm(dim3 grid, hipStream_t s, const void* proj, int width, int q_off, int k_off, int v_off, int gate_off,
                   const float* gate_bias, float cap, float* S, float* n, float* m, float* out, const int32_t* slots,
-                  const int32_t* starts, const int32_t* qs, int heads, int dim, int vdim) {
+                  const int32_t* starts, const int32_t* qs, int heads, int dim, int vdim, int col_blocks, MlstmPieces pc) {
   mlstm_scan_kernel<KD, T><<<grid, WAVE, 0, s>>>((const T*)proj, width, q_off, k_off, v_off, gate_off, gate_bias, cap, S, n,
-                                                  m, out, slots, starts, qs, heads, dim, vdim);
+                                                  m, out, slots, starts, qs, heads, dim, vdim, col_blocks, pc);
 }
 }  // namespace
 
@@ -174,24 +332,55 @@ void launch_mlstm(dim3 grid, hipStream_t s, const void* proj, int width, int q_o
 extern "C" int holon_mlstm_scan(const void* proj, int width, int q_off, int k_off, int v_off, int gate_off,
                                 const float* gate_bias, float cap, float* S, float* n, float* m, float* out,
                                 const int32_t* slots, const int32_t* starts, const int32_t* query_start, int rows,
-                                int heads, int dim, int vdim, int state_slots, int dtype, void* stream) {
+                                int heads, int dim, int vdim, int state_slots, int dtype, int tokens, int piece_tokens,
+                                int max_pieces, const int32_t* piece_base, float* gates, float* sloc, float* nloc,
+                                float* pk, void* stream) {
   HOLON_CHECK(rows >= 0 && heads > 0 && heads <= 65535 && dim > 0 && dim <= 256 && vdim > 0 && state_slots > 0,
               "mlstm_scan: %d heads of %d/%d (keys of at most 256)", heads, dim, vdim);
   HOLON_CHECK(cap > 0.f && width > 0 && q_off >= 0 && k_off >= 0 && v_off >= 0 && gate_off >= 0 &&
                   q_off + heads * dim <= width && k_off + heads * dim <= width && v_off + heads * vdim <= width &&
                   gate_off + 2 * heads <= width,
               "mlstm_scan: columns do not lie within rows of %d", width);
+  HOLON_CHECK(piece_tokens == 0 || (piece_tokens > 0 && max_pieces > 0 && piece_base && gates && sloc && nloc && pk),
+              "mlstm_scan: rows in pieces of %d tokens need the pieces' table and workspaces", piece_tokens);
   if (rows == 0) return 0;
   const int col_blocks = (vdim + COLS - 1) / COLS;
-  HOLON_CHECK(col_blocks <= 65535, "mlstm_scan: values of %d exceed one launch", vdim);
-  const dim3 grid(rows, heads, col_blocks);
   hipStream_t s = (hipStream_t)stream;
+  MlstmPieces pc{piece_tokens, 0, piece_base, gates, sloc, nloc, pk};
+#define MLSTM_SCAN(GRID)                                                                                                \
+  do {                                                                                                                  \
+    if (dtype == HOLON_F32)                                                                                             \
+      MLSTM_BY_KEY(dim, (launch_mlstm<float, KD>(GRID, s, proj, width, q_off, k_off, v_off, gate_off, gate_bias, cap, S, \
+                                                 n, m, out, slots, starts, query_start, heads, dim, vdim, col_blocks,   \
+                                                 pc)));                                                                 \
+    else                                                                                                                \
+      MLSTM_BY_KEY(dim, (launch_mlstm<bf16_t, KD>(GRID, s, proj, width, q_off, k_off, v_off, gate_off, gate_bias, cap,  \
+                                                  S, n, m, out, slots, starts, query_start, heads, dim, vdim,           \
+                                                  col_blocks, pc)));                                                    \
+    HOLON_LAUNCH_OK();                                                                                                  \
+  } while (0)
+  if (piece_tokens == 0) {
+    HOLON_CHECK(col_blocks <= 65535, "mlstm_scan: values of %d exceed one launch", vdim);
+    const dim3 grid(rows, heads, col_blocks);
+    MLSTM_SCAN(grid);
+    return 0;
+  }
+  HOLON_CHECK((int64_t)col_blocks * max_pieces <= 65535, "mlstm_scan: %d pieces a row exceed one launch", max_pieces);
+  (void)tokens;
   if (dtype == HOLON_F32)
-    MLSTM_BY_KEY(dim, (launch_mlstm<float, KD>(grid, s, proj, width, q_off, k_off, v_off, gate_off, gate_bias, cap, S, n,
-                                               m, out, slots, starts, query_start, heads, dim, vdim)));
+    mlstm_gates_kernel<float><<<dim3(rows, heads), WAVE, 0, s>>>((const float*)proj, width, gate_off, gate_bias, cap, m,
+                                                                 gates, slots, starts, query_start, heads, col_blocks);
   else
-    MLSTM_BY_KEY(dim, (launch_mlstm<bf16_t, KD>(grid, s, proj, width, q_off, k_off, v_off, gate_off, gate_bias, cap, S,
-                                                n, m, out, slots, starts, query_start, heads, dim, vdim)));
+    mlstm_gates_kernel<bf16_t><<<dim3(rows, heads), WAVE, 0, s>>>((const bf16_t*)proj, width, gate_off, gate_bias, cap, m,
+                                                                  gates, slots, starts, query_start, heads, col_blocks);
   HOLON_LAUNCH_OK();
+  const dim3 grid(rows, heads, col_blocks * max_pieces);
+  pc.mode = 1;
+  MLSTM_SCAN(grid);
+  mlstm_pieces_kernel<<<dim3(rows, heads), 256, 0, s>>>(S, n, slots, starts, query_start, heads, dim, vdim, col_blocks, pc);
+  HOLON_LAUNCH_OK();
+  pc.mode = 2;
+  MLSTM_SCAN(grid);
+#undef MLSTM_SCAN
   return 0;
 }

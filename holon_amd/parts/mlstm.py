@@ -19,7 +19,7 @@ from ..kernels.registry import KernelOp, register_kernel
 from ..registry import register_part
 from .base import FLOAT32, Build, Part, SlotState
 from .linear import Linear
-from .recurrent import MAX_KEY_DIM, _rows
+from .recurrent import MAX_KEY_DIM, _rows, scan_pieces
 
 _P, _I, _F = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
 _DT = {torch.float32: 0, torch.bfloat16: 1}
@@ -31,11 +31,13 @@ def state_copies(vdim: int) -> int:
 
 
 def mlstm_scan_plain(proj, q_off, k_off, v_off, gate_off, gate_bias, cap, S, n, top, slots, starts, query_start,
-                     n_rows, heads, dim, vdim):
+                     n_rows, heads, dim, vdim, pieces=None):
     """proj [T, width]: q [H D] from column q_off, k [H D] from k_off, v [H V] from v_off, the gates' pre-activations
     [2 H] (input gates, then forget gates) from gate_off; gate_bias [2 H] float32. State per slot: S [H, D, V],
     n [H, C, D], top [H, C], float32, read unless the row starts at position 0, written back; C = ceil(V / 8) equal
-    copies (a kernel's blocks, one for every 8 value columns, each keep their own). -> o [T, H, V] float32."""
+    copies (a kernel's blocks, one for every 8 value columns, each keep their own). -> o [T, H, V] float32. `pieces`
+    (what `scan_pieces` answers, or None) lets a kernel run long rows in pieces side by side; the result is the same
+    but for the order of the sums."""
     t = proj.shape[0]
     pf = proj.float()
     q = pf[:, q_off: q_off + heads * dim].view(t, heads, dim) * dim ** -0.5
@@ -65,7 +67,7 @@ def mlstm_scan_plain(proj, q_off, k_off, v_off, gate_off, gate_bias, cap, S, n, 
 
 
 def _mlstm_scan_hip(launch, proj, q_off, k_off, v_off, gate_off, gate_bias, cap, S, n, top, slots, starts,
-                    query_start, n_rows, heads, dim, vdim):
+                    query_start, n_rows, heads, dim, vdim, pieces=None):
     t, width = proj.shape
     ok = proj.is_cuda and proj.is_contiguous() and proj.dtype in _DT and gate_bias.dtype == torch.float32 \
         and gate_bias.is_contiguous() and gate_bias.shape == (2 * heads,) \
@@ -78,15 +80,23 @@ def _mlstm_scan_hip(launch, proj, q_off, k_off, v_off, gate_off, gate_bias, cap,
     if not ok:
         raise ValueError(f"mlstm_scan: rows {tuple(proj.shape)}, state {tuple(S.shape)} do not fit {heads} heads of "
                          f"{dim}/{vdim} (keys of at most {MAX_KEY_DIM})")
-    out = torch.empty((t, heads, vdim), dtype=torch.float32, device=proj.device)
+    f32 = dict(dtype=torch.float32, device=proj.device)
+    out = torch.empty((t, heads, vdim), **f32)
+    extra = (0, 0, None, None, None, None, None)
+    if pieces is not None:
+        tokens, most, base, total = pieces
+        work = (torch.empty((t, heads, 3), **f32), torch.empty((total, heads, dim, vdim), **f32),
+                torch.empty((total, heads, dim), **f32), torch.empty((total, heads), **f32))
+        extra = (tokens, most, base.data_ptr(), *(w.data_ptr() for w in work))
     launch(proj.data_ptr(), width, q_off, k_off, v_off, gate_off, gate_bias.data_ptr(), float(cap), S.data_ptr(),
            n.data_ptr(), top.data_ptr(), out.data_ptr(), slots.data_ptr(), starts.data_ptr(), query_start.data_ptr(),
-           n_rows, heads, dim, vdim, S.shape[0], _DT[proj.dtype])
+           n_rows, heads, dim, vdim, S.shape[0], _DT[proj.dtype], t, *extra)
     return out
 
 
 register_kernel(KernelOp("mlstm_scan", mlstm_scan_plain, "holon_mlstm_scan",
-                         [_P, _I, _I, _I, _I, _I, _P, _F, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I],
+                         [_P, _I, _I, _I, _I, _I, _P, _F, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P,
+                          _P, _P, _P],
                          _mlstm_scan_hip))
 
 
@@ -153,7 +163,7 @@ class MLSTM(Part):
         st = site.slot_state
         o = k.mlstm_scan(proj, at["q"], at["k"], at["v"], at["gates"], self.gate_bias, self.cap,
                          st[self.prefix + "S"], st[self.prefix + "n"], st[self.prefix + "top"], step.slots, step.starts,
-                         step.query_start, step.n_rows, self.heads, self.dim, self.vdim)
+                         step.query_start, step.n_rows, self.heads, self.dim, self.vdim, scan_pieces(step))
         y = k.gated_out(o, proj[:, at["g"]: at["g"] + hv], self.norm, True, self.eps, self.build.dtype, act="sigmoid")
         return self.o(y)
 

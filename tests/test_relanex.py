@@ -278,6 +278,28 @@ def test_a_far_token_reaches_through_the_memory(tmp_path, device):
 
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["mlstm", "A"])
+def test_long_rows_run_in_pieces(folders, name, dtype, device):
+    """Rows long enough for the memory's scan to cut them into pieces that run side by side: a prompt of 700 tokens
+    whole, then portions of 300 and 290 beside a short request and a decode row, then the rest token by token."""
+    folder = folders[name]
+    vocab = MODELS[name][0]["vocab"]
+    long_ids, short_ids = H.random_ids(700, vocab, 31), H.random_ids(41, vocab, 32)
+    rep = _replayer(folder, device, dtype, 16, cache_tokens=1600, max_model_len=704)
+    got = H.run_trace(rep, H.trace_whole({"long": long_ids}))
+    _check(folder, dtype, {"long": long_ids}, got, f"pieces, whole {dtype}")
+    trace = H.Trace()
+    trace.add([("long", 0, long_ids[:300], [0, 127, 128, 255, 256, 299]), ("short", 0, short_ids[:40], [39])])
+    trace.add([("long", 300, long_ids[300:590], [0, 100, 289]), ("short", 40, short_ids[40:], [0])], end=["short"])
+    for at in range(590, 700):
+        trace.add([("long", at, [long_ids[at]], [0])], end=["long"] if at == 699 else [])
+    got = H.run_trace(rep, trace)
+    _check(folder, dtype, {"long": long_ids, "short": short_ids}, got, f"pieces, portions {dtype}")
+    rep.cache.check()
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_long_decoding(folders, dtype, device):
     """180 tokens one by one after a prompt of 5: many window lengths, many pages given back on the way."""
     folder, page = folders["A-sharp"], 8
@@ -415,6 +437,16 @@ def test_kernels_against_their_plain_forms(dtype):
         o1 = k.mlstm_scan(proj, 0, hd, 2 * hd, 2 * hd + 2 * hv, gb, 12.0, *st1, *rows, 3, heads, d, v)
         o2 = kernel_op("mlstm_scan").plain(proj, 0, hd, 2 * hd, 2 * hd + 2 * hv, gb, 12.0, *st2, *rows, 3, heads, d, v)
         assert _rel(o1, o2) < 1e-5 and all(_rel(a, b) < 1e-5 for a, b in zip(st1, st2))
+        # long rows in pieces of 128 tokens: a row of 700 from a carried state, one of 300 from zero, a decode row
+        long = rn(1001, width).to(dtype)
+        long[:, 2 * hd + 2 * hv:] *= 3
+        rows = (torch.tensor([1, 2, 0], dtype=torch.int32, device=dev), torch.tensor([5, 0, 77], dtype=torch.int32, device=dev),
+                torch.tensor([0, 700, 1000, 1001], dtype=torch.int32, device=dev))
+        cut = (128, 6, torch.tensor([0, 6, 9], dtype=torch.int32, device=dev), 10)
+        st3, st4 = [s.clone() for s in state], [s.clone() for s in state]
+        o3 = k.mlstm_scan(long, 0, hd, 2 * hd, 2 * hd + 2 * hv, gb, 12.0, *st3, *rows, 3, heads, d, v, cut)
+        o4 = kernel_op("mlstm_scan").plain(long, 0, hd, 2 * hd, 2 * hd + 2 * hv, gb, 12.0, *st4, *rows, 3, heads, d, v)
+        assert _rel(o3, o4) < 2e-5 and all(_rel(a, b) < 2e-5 for a, b in zip(st3, st4))
         gate, wn = proj[:, 2 * hd + hv: 2 * hd + 2 * hv], rn(hv).to(dtype)
         assert _rel(k.gated_out(o1, gate, wn, True, 1e-6, dtype, act="sigmoid"),
                     kernel_op("gated_out").plain(o1, gate, wn, True, 1e-6, dtype, act="sigmoid")) < tol
