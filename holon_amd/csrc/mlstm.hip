@@ -120,7 +120,7 @@ __global__ void __launch_bounds__(256) mlstm_pieces_kernel(const float* __restri
   const bool carried = starts[b] > 0;
   const int64_t first = pc.base[b];
   const int cells = dim * vdim;
-  for (int e = threadIdx.x; e < cells + dim; e += 256) {
+  for (int e = blockIdx.z * 256 + threadIdx.x; e < cells + dim; e += gridDim.z * 256) {
     const bool of_n = e >= cells;
     float x = !carried ? 0.f : of_n ? n_all[cell * copies * dim + (e - cells)] : S_all[cell * cells + e];
     for (int p = 0; p < pieces - 1; ++p) {
@@ -377,7 +377,9 @@ extern "C" int holon_mlstm_scan(const void* proj, int width, int q_off, int k_of
   const dim3 grid(rows, heads, col_blocks * max_pieces);
   pc.mode = 1;
   MLSTM_SCAN(grid);
-  mlstm_pieces_kernel<<<dim3(rows, heads), 256, 0, s>>>(S, n, slots, starts, query_start, heads, dim, vdim, col_blocks, pc);
+  const int walkers = (dim * vdim + dim + 1023) / 1024;     // blocks a (row, head): four of its values a thread
+  mlstm_pieces_kernel<<<dim3(rows, heads, walkers), 256, 0, s>>>(S, n, slots, starts, query_start, heads, dim, vdim,
+                                                                 col_blocks, pc);
   HOLON_LAUNCH_OK();
   pc.mode = 2;
   MLSTM_SCAN(grid);
