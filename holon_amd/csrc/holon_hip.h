@@ -272,6 +272,16 @@ int holon_softmax_attention(const void* q, void* out, const void* pages, const i
                             int tokens, int heads, int kv_heads, int dim, int vdim, int page_size, int num_pages,
                             const float* sink, float scale, int window, int dtype, void* stream);
 
+// The latent attention's two latents, side by side in `both` [T, q_rank + kv_rank]: each divided by its root mean square
+// and multiplied by its weight; the first to cq [T, q_rank], the second into the token's page as a key row and as a
+// value column (pages of [2, P * kv_rank]).
+int holon_latent_prepare(const void* both, int tokens, int q_rank, int kv_rank, const void* q_weight,
+                         const void* c_weight, float eps, void* cq, void* pages, const int32_t* write_page,
+                         const int32_t* write_off, int page_size, int num_pages, int dtype, void* stream);
+// y [rows, H, B] = x [rows, H, A] times every head's own w [H, B, A], for steps of up to 16 rows.
+int holon_head_linear_rows(const void* x, const void* w, void* y, int rows, int heads, int A, int B, int dtype,
+                           void* stream);
+
 // -- the matrix memory of xLSTM (mlstm.hip) -------------------------------------------------------------------------------
 // proj [T, width]: q, k [H D] and v [H V] and the gates' pre-activations [2 H] (input, then forget) from the given
 // columns; gate_bias [2 H]; state S [slots, H, D, V], n [slots, H, ceil(V / 8), D], m [slots, H, ceil(V / 8)] (a copy

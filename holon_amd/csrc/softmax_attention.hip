@@ -174,3 +174,111 @@ extern "C" int holon_softmax_attention(const void* q, void* out, const void* pag
   HOLON_LAUNCH_OK();
   return 0;
 }
+
+// -- the latent attention's small steps ---------------------------------------------------------------------------------
+namespace {
+
+// One block a token. `both` [T, q_rank + kv_rank] holds the two latents' projections side by side. Each is divided by
+// its root mean square (eps inside the root) and multiplied by its weight, float32 inside, one rounding: the first goes
+// to `cq` [T, q_rank]; the second is the token's entry in the cache, stored twice in the page it belongs to, as a key
+// (a row of [P, kv_rank]) and as a value (a column of [kv_rank, P]).
+template <typename T>
+__global__ void __launch_bounds__(256) latent_prepare_kernel(const T* __restrict__ both, int q_rank, int kv_rank,
+                                                             const T* __restrict__ q_weight, const T* __restrict__ c_weight,
+                                                             float eps, T* __restrict__ cq, T* __restrict__ pages,
+                                                             const int32_t* __restrict__ write_page,
+                                                             const int32_t* __restrict__ write_off, int page_size,
+                                                             int num_pages) {
+  __shared__ float part[2][4];
+  const int t = blockIdx.x, wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  const T* row = both + (int64_t)t * (q_rank + kv_rank);
+  float sq = 0.f, sc = 0.f;
+  for (int d = threadIdx.x; d < q_rank; d += 256) { const float v = Elem<T>::load(row[d]); sq += v * v; }
+  for (int d = threadIdx.x; d < kv_rank; d += 256) { const float v = Elem<T>::load(row[q_rank + d]); sc += v * v; }
+  sq = wave_sum(sq);
+  sc = wave_sum(sc);
+  if (lane == 0) { part[0][wave] = sq; part[1][wave] = sc; }
+  __syncthreads();
+  const float rq = 1.0f / sqrtf(((part[0][0] + part[0][1]) + (part[0][2] + part[0][3])) / (float)q_rank + eps);
+  const float rc = 1.0f / sqrtf(((part[1][0] + part[1][1]) + (part[1][2] + part[1][3])) / (float)kv_rank + eps);
+  for (int d = threadIdx.x; d < q_rank; d += 256)
+    cq[(int64_t)t * q_rank + d] = Elem<T>::store(Elem<T>::load(row[d]) * rq * Elem<T>::load(q_weight[d]));
+  const int page = write_page[t], off = write_off[t];
+  if (page < 0 || page >= num_pages || off < 0 || off >= page_size) return;
+  T* keys = pages + (int64_t)page * 2 * page_size * kv_rank;
+  T* vals = keys + (int64_t)page_size * kv_rank;
+  for (int d = threadIdx.x; d < kv_rank; d += 256) {
+    const T c = Elem<T>::store(Elem<T>::load(row[q_rank + d]) * rc * Elem<T>::load(c_weight[d]));
+    keys[(int64_t)off * kv_rank + d] = c;
+    vals[(int64_t)d * page_size + off] = c;
+  }
+}
+
+// y[t, h, b] = sum_a x[t, h, a] w[h, b, a] for steps of few rows: a block takes a head and 16 of its output columns,
+// the rows' values of that head wait in LDS, and sixteen lanes share a column (each a sixteenth of A, in the order of
+// the lane), added up in a fixed order. float32 sums, one rounding.
+template <typename T>
+__global__ void __launch_bounds__(256) head_linear_kernel(const T* __restrict__ x, const T* __restrict__ w,
+                                                          T* __restrict__ y, int rows, int heads, int A, int B) {
+  extern __shared__ float xs[];                          // [rows, A]
+  const int h = blockIdx.x, b = blockIdx.y * 16 + threadIdx.x / 16, part = threadIdx.x % 16;
+  for (int i = threadIdx.x; i < rows * A; i += 256) {
+    const int t = i / A, a = i - t * A;
+    xs[i] = Elem<T>::load(x[((int64_t)t * heads + h) * A + a]);
+  }
+  __syncthreads();
+  const T* wr = w + ((int64_t)h * B + (b < B ? b : 0)) * A;
+  for (int t0 = 0; t0 < rows; t0 += 8) {
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    for (int a = part; a < A; a += 16) {
+      const float wv = Elem<T>::load(wr[a]);
+#pragma unroll
+      for (int r = 0; r < 8; ++r)
+        if (t0 + r < rows) acc[r] += xs[(t0 + r) * A + a] * wv;
+    }
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      float v = acc[r];
+      v += __shfl_xor(v, 1, WAVE);
+      v += __shfl_xor(v, 2, WAVE);
+      v += __shfl_xor(v, 4, WAVE);
+      v += __shfl_xor(v, 8, WAVE);
+      if (part == 0 && b < B && t0 + r < rows) y[((int64_t)(t0 + r) * heads + h) * B + b] = Elem<T>::store(v);
+    }
+  }
+}
+}  // namespace
+
+extern "C" int holon_latent_prepare(const void* both, int tokens, int q_rank, int kv_rank, const void* q_weight,
+                                    const void* c_weight, float eps, void* cq, void* pages, const int32_t* write_page,
+                                    const int32_t* write_off, int page_size, int num_pages, int dtype, void* stream) {
+  HOLON_CHECK(tokens >= 0 && q_rank > 0 && kv_rank > 0 && page_size > 0 && num_pages > 0,
+              "latent_prepare: latents of %d and %d, pages of %d", q_rank, kv_rank, page_size);
+  if (tokens == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == HOLON_F32)
+    latent_prepare_kernel<float><<<tokens, 256, 0, s>>>((const float*)both, q_rank, kv_rank, (const float*)q_weight,
+                                                       (const float*)c_weight, eps, (float*)cq, (float*)pages,
+                                                       write_page, write_off, page_size, num_pages);
+  else
+    latent_prepare_kernel<bf16_t><<<tokens, 256, 0, s>>>((const bf16_t*)both, q_rank, kv_rank, (const bf16_t*)q_weight,
+                                                        (const bf16_t*)c_weight, eps, (bf16_t*)cq, (bf16_t*)pages,
+                                                        write_page, write_off, page_size, num_pages);
+  HOLON_LAUNCH_OK();
+  return 0;
+}
+
+extern "C" int holon_head_linear_rows(const void* x, const void* w, void* y, int rows, int heads, int A, int B,
+                                      int dtype, void* stream) {
+  HOLON_CHECK(rows >= 1 && rows <= 16 && heads > 0 && heads <= 65535 && A > 0 && B > 0 && (int64_t)rows * A * 4 <= 48 * 1024,
+              "head_linear (few rows): %d rows, %d heads of %d -> %d", rows, heads, A, B);
+  const dim3 grid(heads, (B + 15) / 16);
+  const size_t lds = (size_t)rows * A * sizeof(float);
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == HOLON_F32)
+    head_linear_kernel<float><<<grid, 256, lds, s>>>((const float*)x, (const float*)w, (float*)y, rows, heads, A, B);
+  else
+    head_linear_kernel<bf16_t><<<grid, 256, lds, s>>>((const bf16_t*)x, (const bf16_t*)w, (bf16_t*)y, rows, heads, A, B);
+  HOLON_LAUNCH_OK();
+  return 0;
+}

@@ -78,15 +78,66 @@ def _softmax_attention_hip(launch, q, pages, table, rows, token_row, positions, 
 
 
 def head_linear_plain(x, weight):
-    """x [T, H, A], weight [H, B, A] -> [T, H, B]: every head's own small projection (a batched matrix product, the
-    vendor library's on the GPU), sums in float32, the result in x's dtype."""
+    """x [T, H, A], weight [H, B, A] -> [T, H, B]: every head's own small projection, sums in float32, the result in
+    x's dtype."""
     return torch.einsum("tha,hba->thb", x, weight.to(x.dtype)).contiguous()
+
+
+def _head_linear_hip(launch, x, weight):
+    """Steps of up to 16 rows: this package's kernel (the weights stream once, no copy of the result); more rows: the
+    vendor library's batched product."""
+    t, heads, a = x.shape
+    b = weight.shape[1]
+    if not (x.is_cuda and x.is_contiguous() and weight.is_contiguous() and weight.dtype == x.dtype and x.dtype in _DT
+            and tuple(weight.shape) == (heads, b, a)):
+        raise ValueError(f"head_linear: rows {tuple(x.shape)} {x.dtype} do not fit weights {tuple(weight.shape)} {weight.dtype}")
+    if not 1 <= t <= 16 or t * a * 4 > 48 * 1024:
+        return head_linear_plain(x, weight)
+    y = torch.empty((t, heads, b), dtype=x.dtype, device=x.device)
+    launch(x.data_ptr(), weight.data_ptr(), y.data_ptr(), t, heads, a, b, _DT[x.dtype])
+    return y
+
+
+def latent_prepare_plain(both, q_rank, q_weight, c_weight, eps, pages, write_page, write_off, page_size):
+    """both [T, q_rank + R] (the two latents' projections side by side): each x * rsqrt(mean(x^2) + eps) * weight,
+    float32 inside, one rounding. Returns the first [T, q_rank]; the second goes into `pages` [pages, 2 P R] at
+    (write_page[t], write_off[t]) twice: as a key (row of [P, R]) and as a value (column of [R, P])."""
+    t, rank = both.shape[0], both.shape[1] - q_rank
+
+    def norm(x, w):
+        xf = x.float()
+        return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps) * w.float()).to(both.dtype)
+    cq, c = norm(both[:, :q_rank], q_weight), norm(both[:, q_rank:], c_weight)
+    keys = pages[:, : page_size * rank].view(-1, page_size, rank)
+    vals = pages[:, page_size * rank:].view(-1, rank, page_size)
+    keys[write_page.long(), write_off.long()] = c
+    vals[write_page.long(), :, write_off.long()] = c
+    return cq.contiguous()
+
+
+def _latent_prepare_hip(launch, both, q_rank, q_weight, c_weight, eps, pages, write_page, write_off, page_size):
+    t, rank = both.shape[0], both.shape[1] - q_rank
+    ok = both.is_cuda and both.is_contiguous() and both.dtype in _DT and rank > 0 and pages.dtype == both.dtype \
+        and pages.is_contiguous() and pages.dim() == 2 and pages.shape[1] == 2 * page_size * rank \
+        and all(w.dtype == both.dtype and w.is_contiguous() for w in (q_weight, c_weight)) \
+        and q_weight.shape == (q_rank,) and c_weight.shape == (rank,) and write_page.shape[0] >= t \
+        and write_off.shape[0] >= t
+    if not ok:
+        raise ValueError(f"latent_prepare: rows {tuple(both.shape)} {both.dtype}, pages {tuple(pages.shape)} do not fit "
+                         f"latents of {q_rank} and {rank}, page {page_size}")
+    cq = torch.empty((t, q_rank), dtype=both.dtype, device=both.device)
+    launch(both.data_ptr(), t, q_rank, rank, q_weight.data_ptr(), c_weight.data_ptr(), float(eps), cq.data_ptr(),
+           pages.data_ptr(), write_page.data_ptr(), write_off.data_ptr(), page_size, pages.shape[0], _DT[both.dtype])
+    return cq
 
 
 register_kernel(KernelOp("softmax_attention", softmax_attention_plain, "holon_softmax_attention",
                          [_P, _P, _P, _P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P, _F, _I, _I],
                          _softmax_attention_hip))
-register_kernel(KernelOp("head_linear", head_linear_plain))
+register_kernel(KernelOp("head_linear", head_linear_plain, "holon_head_linear_rows", [_P, _P, _P, _I, _I, _I, _I, _I],
+                         _head_linear_hip))
+register_kernel(KernelOp("latent_prepare", latent_prepare_plain, "holon_latent_prepare",
+                         [_P, _I, _I, _I, _P, _P, _F, _P, _P, _P, _P, _I, _I, _I], _latent_prepare_hip))
 
 
 def attend(k, q, held, view, step, kv_heads, vdim, sink, scale, window):
@@ -211,6 +262,8 @@ class LatentAttention(Part):
         self.attach("o", Linear(build, inp=heads * vdim, out=hidden))
         self.down: Linear | None = None
         self.uk_t = self.uv_h = None
+        self._fused: float | None = None          # the norms' eps, when they are RMS norms of one eps: one kernel then
+                                                  # norms both latents and writes the cache
 
     def state(self):
         return [PagedState(self.state_name, elems=2 * self.kv_rank, window=self.window)]
@@ -220,6 +273,10 @@ class LatentAttention(Part):
         self.drop("dq")
         self.drop("dkv")
         self._children["down"] = self.down
+        specs = [n.fusion() for n in (self.dq_norm, self.dkv_norm)]
+        if all(sp is not None and sp.get("norm") == "rmsnorm" and sp["weight"] is not None for sp in specs) \
+                and specs[0]["eps"] == specs[1]["eps"]:
+            self._fused = float(specs[0]["eps"])
         if self.uk is not None:
             # [H, kv_rank, dim]: what turns a head's query into the latent's space; [H, vdim, kv_rank]: a head's values
             self.uk_t = self.uk.view(self.heads, self.dim, self.kv_rank).transpose(1, 2).contiguous()
@@ -234,10 +291,14 @@ class LatentAttention(Part):
         held = site.paged[self.state_name]
         view = step.paged[held.group]
         both = self.down(x)
-        cq = self.dq_norm(both[:, : self.q_rank].contiguous())
-        c = self.dkv_norm(both[:, self.q_rank:].contiguous()).view(t, 1, self.kv_rank)
-        k.kv_write(c, c, held.pages.view(-1, 2, 1, view.page_size * self.kv_rank), view.write_page, view.write_off,
-                   view.page_size)
+        if self._fused is not None:               # both norms and the cache write in one kernel
+            cq = k.latent_prepare(both, self.q_rank, self.dq_norm.weight, self.dkv_norm.weight, self._fused, held.pages,
+                                  view.write_page, view.write_off, view.page_size)
+        else:
+            cq = self.dq_norm(both[:, : self.q_rank].contiguous())
+            c = self.dkv_norm(both[:, self.q_rank:].contiguous()).view(t, 1, self.kv_rank)
+            k.kv_write(c, c, held.pages.view(-1, 2, 1, view.page_size * self.kv_rank), view.write_page, view.write_off,
+                       view.page_size)
         q = k.head_linear(self.uq(cq).view(t, self.heads, self.dim), self.uk_t)
         mixed = attend(k, q, held, view, step, 1, self.kv_rank, None, self.scale, self.window)
         out = k.head_linear(mixed.view(t, self.heads, self.kv_rank), self.uv_h)

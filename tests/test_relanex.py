@@ -423,6 +423,19 @@ def test_kernels_against_their_plain_forms(dtype):
     q2 = kernel_op("head_prepare").plain(qkv, heads, kv, d, v, None, None, 0.0, tab, pos, pg2, pos // page, pos % page,
                                          page, bias=bias)
     assert _rel(q1, q2) < tol and _rel(pg1, pg2) < tol
+    for t, heads, a, b in ((1, 6, 32, 96), (8, 16, 128, 256), (16, 3, 96, 80), (5, 2, 24, 7), (40, 4, 64, 48)):
+        x, w = rn(t, heads, a).to(dtype), (rn(heads, b, a) * a ** -0.5).to(dtype)      # every head's own projection
+        assert _rel(k.head_linear(x, w), kernel_op("head_linear").plain(x.float(), w.float())) < tol
+    for q_rank, rank, page in ((96, 96, 16), (24, 40, 8), (768, 256, 16), (7, 5, 4)):       # the two latents' norms
+        t = 21
+        both, qw, cw = rn(t, q_rank + rank).to(dtype), (1 + 0.1 * rn(q_rank)).to(dtype), (1 + 0.1 * rn(rank)).to(dtype)
+        pos = torch.arange(t, dtype=torch.int32, device=dev)
+        pg1 = torch.zeros((t + 3) // page + 1, 2 * page * rank, device=dev, dtype=dtype)      # every token's page exists
+        pg2 = pg1.clone()
+        wp, wo = (pos + 3) // page, (pos + 3) % page
+        c1 = k.latent_prepare(both, q_rank, qw, cw, 1e-6, pg1, wp, wo, page)
+        c2 = kernel_op("latent_prepare").plain(both, q_rank, qw, cw, 1e-6, pg2, wp, wo, page)
+        assert _rel(c1, c2) < tol and _rel(pg1, pg2) < tol
     for heads, d, v in ((4, 48, 48), (2, 16, 40), (3, 64, 8), (1, 128, 20), (2, 200, 16)):     # the memory's scan
         hd, hv, copies = heads * d, heads * v, -(-v // 8)
         width = -(-(2 * hd + 2 * hv + 2 * heads) // 16) * 16
