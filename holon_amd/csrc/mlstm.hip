@@ -271,16 +271,16 @@ __global__ void __launch_bounds__(WAVE) mlstm_scan_kernel(const T* __restrict__ 
         pk *= keep;
         continue;
       }
-      float o = 0.f, d = 0.f;
+      float os[4] = {0.f, 0.f, 0.f, 0.f}, ds[4] = {0.f, 0.f, 0.f, 0.f};     // four short chains of sums, not one long one
 #pragma unroll
       for (int i = 0; i < KQ; ++i) {
         S[i] = keep * S[i] + kt[i] * vt;
         nn[i] = keep * nn[i] + take * kt[i];
-        o += S[i] * qt[i];
-        d += nn[i] * qt[i];
+        os[i % 4] += S[i] * qt[i];
+        ds[i % 4] += nn[i] * qt[i];
       }
-      o = part_sum(o);
-      d = part_sum(d);
+      const float o = part_sum((os[0] + os[1]) + (os[2] + os[3]));
+      const float d = part_sum((ds[0] + ds[1]) + (ds[2] + ds[3]));
       const float den = fmaxf(fabsf(d), floor_) + 1e-6f;
       if (active && part == 0) out[((int64_t)(t0 + tt) * heads + h) * vdim + j] = o / den;
     }

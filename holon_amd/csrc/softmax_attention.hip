@@ -228,13 +228,32 @@ __global__ void __launch_bounds__(256) head_linear_kernel(const T* __restrict__ 
   }
   __syncthreads();
   const T* wr = w + ((int64_t)h * B + (b < B ? b : 0)) * A;
+  constexpr int VEC = Elem<T>::kVec;
+  const bool wide = A % (16 * VEC) == 0 && (uintptr_t)w % 16 == 0;      // a lane's share as 16-byte loads
   for (int t0 = 0; t0 < rows; t0 += 8) {
     float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    for (int a = part; a < A; a += 16) {
-      const float wv = Elem<T>::load(wr[a]);
+    if (wide) {
+      for (int a = part * VEC; a < A; a += 16 * VEC) {
+        const uint4 raw = *reinterpret_cast<const uint4*>(wr + a);
+        const T* e = reinterpret_cast<const T*>(&raw);
+        float wv[VEC];
 #pragma unroll
-      for (int r = 0; r < 8; ++r)
-        if (t0 + r < rows) acc[r] += xs[(t0 + r) * A + a] * wv;
+        for (int i = 0; i < VEC; ++i) wv[i] = Elem<T>::load(e[i]);
+#pragma unroll
+        for (int r = 0; r < 8; ++r)
+          if (t0 + r < rows) {
+            const float* xr = xs + (t0 + r) * A + a;
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) acc[r] += xr[i] * wv[i];
+          }
+      }
+    } else {
+      for (int a = part; a < A; a += 16) {
+        const float wv = Elem<T>::load(wr[a]);
+#pragma unroll
+        for (int r = 0; r < 8; ++r)
+          if (t0 + r < rows) acc[r] += xs[(t0 + r) * A + a] * wv;
+      }
     }
 #pragma unroll
     for (int r = 0; r < 8; ++r) {
