@@ -222,9 +222,11 @@ int holon_memory_scan(const void* r, const void* k, const void* v, const float* 
                       int heads, int dim, int state_slots, int dtype, int piece_tokens, int max_pieces,
                       const int32_t* piece_base, float* sloc, float* pw, void* stream);
 // y [T, H V] = o / sqrt(mean_V(o^2) + eps) * weight * act(gate); weight [V], or [H V] with per_head; act is silu, or
-// with plain_sigmoid the sigmoid alone; a token's H V gates start gate_stride values after the token before's.
+// with plain_sigmoid the sigmoid alone; a token's H V gates start gate_stride values after the token before's. den
+// [T, H] float32 or NULL: every head's o is divided by it first.
 int holon_gated_out(const float* o, const void* gate, const void* weight, void* y, int tokens, int heads, int vdim,
-                    int per_head, float eps, int dtype, int64_t gate_stride, int plain_sigmoid, void* stream);
+                    int per_head, float eps, int dtype, int64_t gate_stride, int plain_sigmoid, const float* den,
+                    void* stream);
 // y [mixes, T, W] = x + (x' - x) mu_s, x' the row of the token before (state [state_slots, W] for a row's first
 // token, zeros for a row that starts at 0); the state then takes each row's last x.
 int holon_shift_mix(const void* x, const void* mu, void* state, void* y, const int32_t* slots, const int32_t* starts,
@@ -284,15 +286,16 @@ int holon_head_linear_rows(const void* x, const void* w, void* y, int rows, int 
 
 // -- the matrix memory of xLSTM (mlstm.hip) -------------------------------------------------------------------------------
 // proj [T, width]: q, k [H D] and v [H V] and the gates' pre-activations [2 H] (input, then forget) from the given
-// columns; gate_bias [2 H]; state S [slots, H, D, V], n [slots, H, ceil(V / 8), D], m [slots, H, ceil(V / 8)] (a copy
-// for every 8 value columns), float32; out [T, H, V] float32. piece_tokens > 0: rows are cut into pieces of that many
-// tokens that run side by side in two passes (at most max_pieces a row; piece_base [rows]: the number of each row's
-// first piece among all; workspaces gates [T, H, 3], sloc [pieces, H, D, V], nloc [pieces, H, D], pk [pieces, H]).
+// columns; gate_bias [2 H]; state S [slots, H, D, V + 1] (the last column is n) and m [slots, H, ceil((V + 1) / 8)] (a
+// copy for every 8 columns), float32; out [T, H, V] the numerators S^T q and den [T, H] the denominators
+// max(|n . q|, exp(-m)) + 1e-6, float32. piece_tokens > 0: rows are cut into pieces of that many tokens that run side
+// by side in two passes (at most max_pieces a row; piece_base [rows]: the number of each row's first piece among all;
+// workspaces gates [T, H, 3], sloc [pieces, H, D, V + 1], pk [pieces, H]).
 int holon_mlstm_scan(const void* proj, int width, int q_off, int k_off, int v_off, int gate_off, const float* gate_bias,
-                     float cap, float* S, float* n, float* m, float* out, const int32_t* slots, const int32_t* starts,
+                     float cap, float* S, float* m, float* out, float* den, const int32_t* slots, const int32_t* starts,
                      const int32_t* query_start, int rows, int heads, int dim, int vdim, int state_slots, int dtype,
                      int tokens, int piece_tokens, int max_pieces, const int32_t* piece_base, float* gates, float* sloc,
-                     float* nloc, float* pk, void* stream);
+                     float* pk, void* stream);
 
 #ifdef __cplusplus
 }

@@ -7,12 +7,14 @@
 // f = logsigmoid(cap tanh((a_f + b_f) / cap)); q is scaled by D^-0.5. q, k, v and the gates are columns of one
 // projection's rows.
 //
-// S's columns never meet, so a wave owns 8 of them, eight lanes a column with an eighth of the key rows each (n's rows
-// likewise, held again by every column); what a token needs of a whole column is summed over a lane's rows in ascending
-// order and then over the eight lanes in a fixed order. A batch of tokens' operands travels from memory to LDS while
+// n is kept as one more column of S (the column of a value that is always 1), so the state is S [D, V + 1] and the
+// kernel leaves the numerators S'^T q [V] and the denominator max(|n' . q|, exp(-m')) + 1e-6 of every token; the
+// read-out kernel that follows divides. S's columns never meet, so a wave owns 8 of them, eight lanes a column with an
+// eighth of the key rows each; what a token needs of a whole column is summed over a lane's rows in four interleaved
+// chains and then over the eight lanes in a fixed order. A batch of tokens' operands travels from memory to LDS while
 // the batch before is worked through; the gates' functions are taken then, off the recurrence's path.
-// The blocks of a head (one for every 8 columns) all need n and m and do not wait for each other, so each keeps a copy
-// of its own in the slot, n [H, V/8, D] and m [H, V/8]: a block reads and writes nothing that another block touches.
+// The blocks of a head (one for every 8 columns) all need m and do not wait for each other, so each keeps a copy of
+// its own in the slot, m [H, ceil((V + 1) / 8)]: a block reads and writes nothing that another block touches.
 //
 // Long rows run in pieces side by side. The maxima depend on the gates alone, m' = max(m + f, i), a recurrence whose
 // steps compose ((a, b) then (c, d) is (a + c, max(b + c, d))), so a wave finds a whole row's maxima by a prefix scan and
@@ -47,8 +49,7 @@ struct MlstmPieces {
   int mode;                    // 1: from zero, leave what the piece adds; 2: from the true start, write outputs
   const int32_t* base;         // [rows]: the number of row b's first piece among all pieces of the step
   const float* gates;          // [T, H, 3]: exp(f + m - m'), exp(i - m'), exp(-m') of every token
-  float* sloc;                 // [pieces, H, D, V]
-  float* nloc;                 // [pieces, H, D]
+  float* sloc;                 // [pieces, H, D, V + 1]
   float* pk;                   // [pieces, H]
 };
 
@@ -106,12 +107,12 @@ __global__ void __launch_bounds__(WAVE) mlstm_gates_kernel(const T* __restrict__
     for (int c = 0; c < copies; ++c) m_all[cell + c] = m;
 }
 
-// A row's pieces in order: S <- pk S + sloc (n likewise); sloc[p] becomes the state piece p + 1 starts from.
-__global__ void __launch_bounds__(256) mlstm_pieces_kernel(const float* __restrict__ S_all, const float* __restrict__ n_all,
+// A row's pieces in order: S <- pk S + sloc; sloc[p] becomes the state piece p + 1 starts from.
+__global__ void __launch_bounds__(256) mlstm_pieces_kernel(const float* __restrict__ S_all,
                                                            const int32_t* __restrict__ slots,
                                                            const int32_t* __restrict__ starts,
-                                                           const int32_t* __restrict__ query_start, int heads, int dim,
-                                                           int vdim, int copies, MlstmPieces pc) {
+                                                           const int32_t* __restrict__ query_start, int heads, int cells,
+                                                           MlstmPieces pc) {
   const int b = blockIdx.x, h = blockIdx.y;
   const int n = query_start[b + 1] - query_start[b];
   const int pieces = (n + pc.tokens - 1) / pc.tokens;
@@ -119,13 +120,11 @@ __global__ void __launch_bounds__(256) mlstm_pieces_kernel(const float* __restri
   const int64_t cell = (int64_t)slots[b] * heads + h;
   const bool carried = starts[b] > 0;
   const int64_t first = pc.base[b];
-  const int cells = dim * vdim;
-  for (int e = blockIdx.z * 256 + threadIdx.x; e < cells + dim; e += gridDim.z * 256) {
-    const bool of_n = e >= cells;
-    float x = !carried ? 0.f : of_n ? n_all[cell * copies * dim + (e - cells)] : S_all[cell * cells + e];
+  for (int e = blockIdx.z * 256 + threadIdx.x; e < cells; e += gridDim.z * 256) {
+    float x = carried ? S_all[cell * cells + e] : 0.f;
     for (int p = 0; p < pieces - 1; ++p) {
       const int64_t at = (first + p) * heads + h;
-      float* add = of_n ? pc.nloc + at * dim + (e - cells) : pc.sloc + at * cells + e;
+      float* add = pc.sloc + at * cells + e;
       x = pc.pk[at] * x + *add;
       *add = x;
     }
@@ -135,8 +134,8 @@ __global__ void __launch_bounds__(256) mlstm_pieces_kernel(const float* __restri
 template <int KD, typename T>
 __global__ void __launch_bounds__(WAVE) mlstm_scan_kernel(const T* __restrict__ proj, int width, int q_off, int k_off,
                                                           int v_off, int gate_off, const float* __restrict__ gate_bias,
-                                                          float cap, float* __restrict__ S_all, float* __restrict__ n_all,
-                                                          float* __restrict__ m_all, float* __restrict__ out,
+                                                          float cap, float* __restrict__ S_all, float* __restrict__ m_all,
+                                                          float* __restrict__ out, float* __restrict__ den_out,
                                                           const int32_t* __restrict__ slots,
                                                           const int32_t* __restrict__ starts,
                                                           const int32_t* __restrict__ query_start, int heads, int dim,
@@ -147,7 +146,8 @@ __global__ void __launch_bounds__(WAVE) mlstm_scan_kernel(const T* __restrict__ 
   const int b = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int piece = blockIdx.z / col_blocks, col_block = blockIdx.z % col_blocks;
   const int part = lane % PARTS, col = lane / PARTS, j = col_block * COLS + col;
-  const bool active = j < vdim;
+  const int cols = vdim + 1;                           // S's columns: the values', then n's
+  const bool active = j < cols, of_n = j == vdim;
   int lo = query_start[b], hi = query_start[b + 1];
   const bool cut = pc.tokens > 0;                      // (the gates then come as factors: gi = keep, gf = take, ge = exp(-m))
   bool from_slot = true, to_slot = true;
@@ -163,23 +163,20 @@ __global__ void __launch_bounds__(WAVE) mlstm_scan_kernel(const T* __restrict__ 
   }
   const bool local = cut && pc.mode == 1;
   const int64_t cell = (int64_t)slots[b] * heads + h;
-  const int64_t mine = cell * col_blocks + col_block;        // this block's own copy of n and m
-  float* S_held = S_all + cell * dim * vdim;
-  float* n_held = n_all + mine * dim;
+  const int64_t mine = cell * col_blocks + col_block;        // this block's own copy of m
+  float* S_held = S_all + cell * dim * cols;
   const bool carried = starts[b] > 0;
-  float S[KQ], nn[KQ];
+  float S[KQ];
 #pragma unroll
   for (int i = 0; i < KQ; ++i) {
     const int row = part * KQ + i;
     if (local) {
-      S[i] = nn[i] = 0.f;
+      S[i] = 0.f;
     } else if (from_slot) {
-      S[i] = (carried && active && row < dim) ? S_held[(int64_t)row * vdim + j] : 0.f;
-      nn[i] = (carried && row < dim) ? n_held[row] : 0.f;
+      S[i] = (carried && active && row < dim) ? S_held[(int64_t)row * cols + j] : 0.f;
     } else {
       const int64_t at = (piece_no - 1) * heads + h;
-      S[i] = (active && row < dim) ? pc.sloc[at * dim * vdim + (int64_t)row * vdim + j] : 0.f;
-      nn[i] = row < dim ? pc.nloc[at * dim + row] : 0.f;
+      S[i] = (active && row < dim) ? pc.sloc[at * dim * cols + (int64_t)row * cols + j] : 0.f;
     }
   }
   float m = (carried && !cut) ? m_all[mine] : 0.f;
@@ -217,7 +214,7 @@ __global__ void __launch_bounds__(WAVE) mlstm_scan_kernel(const T* __restrict__ 
     for (int e = 0; e < 2; ++e) {
       const int idx = lane + e * WAVE, tt = idx / COLS, jj = col_block * COLS + idx % COLS;
       const bool ok = idx < TC * COLS && t0 + tt < hi && jj < vdim;
-      nv2[e] = ok ? Elem<T>::load(proj[(int64_t)(t0 + tt) * width + v_off + h * vdim + jj]) : 0.f;
+      nv2[e] = ok ? Elem<T>::load(proj[(int64_t)(t0 + tt) * width + v_off + h * vdim + jj]) : (jj == vdim ? 1.f : 0.f);
     }
   };
   auto put = [&](int buf) {
@@ -264,25 +261,21 @@ __global__ void __launch_bounds__(WAVE) mlstm_scan_kernel(const T* __restrict__ 
       const float* kt = &ks[buf][tt * KD + part * KQ];
       if (local) {                       // what the piece adds, and the product of its factors; no output yet
 #pragma unroll
-        for (int i = 0; i < KQ; ++i) {
-          S[i] = keep * S[i] + kt[i] * vt;
-          nn[i] = keep * nn[i] + take * kt[i];
-        }
+        for (int i = 0; i < KQ; ++i) S[i] = keep * S[i] + kt[i] * vt;
         pk *= keep;
         continue;
       }
-      float os[4] = {0.f, 0.f, 0.f, 0.f}, ds[4] = {0.f, 0.f, 0.f, 0.f};     // four short chains of sums, not one long one
+      float os[4] = {0.f, 0.f, 0.f, 0.f};              // four short chains of sums, not one long one
 #pragma unroll
       for (int i = 0; i < KQ; ++i) {
         S[i] = keep * S[i] + kt[i] * vt;
-        nn[i] = keep * nn[i] + take * kt[i];
         os[i % 4] += S[i] * qt[i];
-        ds[i % 4] += nn[i] * qt[i];
       }
       const float o = part_sum((os[0] + os[1]) + (os[2] + os[3]));
-      const float d = part_sum((ds[0] + ds[1]) + (ds[2] + ds[3]));
-      const float den = fmaxf(fabsf(d), floor_) + 1e-6f;
-      if (active && part == 0) out[((int64_t)(t0 + tt) * heads + h) * vdim + j] = o / den;
+      if (active && part == 0) {
+        if (of_n) den_out[(int64_t)(t0 + tt) * heads + h] = fmaxf(fabsf(o), floor_) + 1e-6f;
+        else out[((int64_t)(t0 + tt) * heads + h) * vdim + j] = o;
+      }
     }
     if (t0 + TC < hi) put(buf ^ 1);
     __syncthreads();
@@ -294,8 +287,7 @@ __global__ void __launch_bounds__(WAVE) mlstm_scan_kernel(const T* __restrict__ 
     for (int i = 0; i < KQ; ++i) {
       const int row = part * KQ + i;
       if (row >= dim) continue;
-      if (active) pc.sloc[at * dim * vdim + (int64_t)row * vdim + j] = S[i];
-      if (col_block == 0 && col == 0) pc.nloc[at * dim + row] = nn[i];
+      if (active) pc.sloc[at * dim * cols + (int64_t)row * cols + j] = S[i];
     }
     if (col_block == 0 && lane == 0) pc.pk[at] = pk;
     return;
@@ -305,18 +297,17 @@ __global__ void __launch_bounds__(WAVE) mlstm_scan_kernel(const T* __restrict__ 
   for (int i = 0; i < KQ; ++i) {
     const int row = part * KQ + i;
     if (row >= dim) continue;
-    if (active) S_held[(int64_t)row * vdim + j] = S[i];
-    if (col == 0) n_held[row] = nn[i];
+    if (active) S_held[(int64_t)row * cols + j] = S[i];
   }
   if (lane == 0 && !cut) m_all[mine] = m;              // (cut: the gates' kernel has left the row's last maximum)
 }
 
 template <typename T, int KD>
 void launch_mlstm(dim3 grid, hipStream_t s, const void* proj, int width, int q_off, int k_off, int v_off, int gate_off,
-                  const float* gate_bias, float cap, float* S, float* n, float* m, float* out, const int32_t* slots,
+                  const float* gate_bias, float cap, float* S, float* m, float* out, float* den, const int32_t* slots,
                   const int32_t* starts, const int32_t* qs, int heads, int dim, int vdim, int col_blocks, MlstmPieces pc) {
-  mlstm_scan_kernel<KD, T><<<grid, WAVE, 0, s>>>((const T*)proj, width, q_off, k_off, v_off, gate_off, gate_bias, cap, S, n,
-                                                  m, out, slots, starts, qs, heads, dim, vdim, col_blocks, pc);
+  mlstm_scan_kernel<KD, T><<<grid, WAVE, 0, s>>>((const T*)proj, width, q_off, k_off, v_off, gate_off, gate_bias, cap, S, m,
+                                                  out, den, slots, starts, qs, heads, dim, vdim, col_blocks, pc);
 }
 }  // namespace
 
@@ -330,32 +321,32 @@ void launch_mlstm(dim3 grid, hipStream_t s, const void* proj, int width, int q_o
   } while (0)
 
 extern "C" int holon_mlstm_scan(const void* proj, int width, int q_off, int k_off, int v_off, int gate_off,
-                                const float* gate_bias, float cap, float* S, float* n, float* m, float* out,
+                                const float* gate_bias, float cap, float* S, float* m, float* out, float* den,
                                 const int32_t* slots, const int32_t* starts, const int32_t* query_start, int rows,
                                 int heads, int dim, int vdim, int state_slots, int dtype, int tokens, int piece_tokens,
-                                int max_pieces, const int32_t* piece_base, float* gates, float* sloc, float* nloc,
-                                float* pk, void* stream) {
+                                int max_pieces, const int32_t* piece_base, float* gates, float* sloc, float* pk,
+                                void* stream) {
   HOLON_CHECK(rows >= 0 && heads > 0 && heads <= 65535 && dim > 0 && dim <= 256 && vdim > 0 && state_slots > 0,
               "mlstm_scan: %d heads of %d/%d (keys of at most 256)", heads, dim, vdim);
   HOLON_CHECK(cap > 0.f && width > 0 && q_off >= 0 && k_off >= 0 && v_off >= 0 && gate_off >= 0 &&
                   q_off + heads * dim <= width && k_off + heads * dim <= width && v_off + heads * vdim <= width &&
                   gate_off + 2 * heads <= width,
               "mlstm_scan: columns do not lie within rows of %d", width);
-  HOLON_CHECK(piece_tokens == 0 || (piece_tokens > 0 && max_pieces > 0 && piece_base && gates && sloc && nloc && pk),
+  HOLON_CHECK(piece_tokens == 0 || (piece_tokens > 0 && max_pieces > 0 && piece_base && gates && sloc && pk),
               "mlstm_scan: rows in pieces of %d tokens need the pieces' table and workspaces", piece_tokens);
   if (rows == 0) return 0;
-  const int col_blocks = (vdim + COLS - 1) / COLS;
+  const int col_blocks = (vdim + 1 + COLS - 1) / COLS;     // the values' columns and n's
   hipStream_t s = (hipStream_t)stream;
-  MlstmPieces pc{piece_tokens, 0, piece_base, gates, sloc, nloc, pk};
+  MlstmPieces pc{piece_tokens, 0, piece_base, gates, sloc, pk};
 #define MLSTM_SCAN(GRID)                                                                                                \
   do {                                                                                                                  \
     if (dtype == HOLON_F32)                                                                                             \
       MLSTM_BY_KEY(dim, (launch_mlstm<float, KD>(GRID, s, proj, width, q_off, k_off, v_off, gate_off, gate_bias, cap, S, \
-                                                 n, m, out, slots, starts, query_start, heads, dim, vdim, col_blocks,   \
+                                                 m, out, den, slots, starts, query_start, heads, dim, vdim, col_blocks, \
                                                  pc)));                                                                 \
     else                                                                                                                \
       MLSTM_BY_KEY(dim, (launch_mlstm<bf16_t, KD>(GRID, s, proj, width, q_off, k_off, v_off, gate_off, gate_bias, cap,  \
-                                                  S, n, m, out, slots, starts, query_start, heads, dim, vdim,           \
+                                                  S, m, out, den, slots, starts, query_start, heads, dim, vdim,         \
                                                   col_blocks, pc)));                                                    \
     HOLON_LAUNCH_OK();                                                                                                  \
   } while (0)
@@ -377,9 +368,9 @@ extern "C" int holon_mlstm_scan(const void* proj, int width, int q_off, int k_of
   const dim3 grid(rows, heads, col_blocks * max_pieces);
   pc.mode = 1;
   MLSTM_SCAN(grid);
-  const int walkers = (dim * vdim + dim + 1023) / 1024;     // blocks a (row, head): four of its values a thread
-  mlstm_pieces_kernel<<<dim3(rows, heads, walkers), 256, 0, s>>>(S, n, slots, starts, query_start, heads, dim, vdim,
-                                                                 col_blocks, pc);
+  const int cells = dim * (vdim + 1);
+  const int walkers = (cells + 1023) / 1024;                // blocks a (row, head): four of its values a thread
+  mlstm_pieces_kernel<<<dim3(rows, heads, walkers), 256, 0, s>>>(S, slots, starts, query_start, heads, cells, pc);
   HOLON_LAUNCH_OK();
   pc.mode = 2;
   MLSTM_SCAN(grid);

@@ -487,26 +487,32 @@ __global__ void __launch_bounds__(256) memory_pieces_kernel(const float* __restr
 }
 
 // One wave per (token, head): o / sqrt(mean(o^2) + eps) * weight * act(gate), act = silu, or the sigmoid alone
-// (`plain_sigmoid`). A token's gates are `gate_stride` values apart (columns of a wider projection).
+// (`plain_sigmoid`). A token's gates are `gate_stride` values apart (columns of a wider projection). With `den`
+// (one value a token and head) o is divided by it first.
 template <typename T>
 __global__ void __launch_bounds__(256) gated_out_kernel(const float* __restrict__ o, const T* __restrict__ gate,
                                                         const T* __restrict__ weight, T* __restrict__ y, int64_t cells,
                                                         int heads, int vdim, int per_head, float eps,
-                                                        int64_t gate_stride, int plain_sigmoid) {
+                                                        int64_t gate_stride, int plain_sigmoid,
+                                                        const float* __restrict__ den) {
   const int64_t cell = (int64_t)blockIdx.x * 4 + threadIdx.x / WAVE;
   const int lane = threadIdx.x % WAVE;
   if (cell >= cells) return;
   const int h = (int)(cell % heads);
   const float* src = o + cell * vdim;
+  const float under = den ? den[cell] : 1.f;
   float ss = 0.f;
-  for (int d = lane; d < vdim; d += WAVE) ss += src[d] * src[d];
+  for (int d = lane; d < vdim; d += WAVE) {
+    const float v = den ? src[d] / under : src[d];
+    ss += v * v;
+  }
   ss = wave_sum(ss);
   const float r = 1.0f / sqrtf(ss / (float)vdim + eps);
   for (int d = lane; d < vdim; d += WAVE) {
     const float wv = Elem<T>::load(weight[per_head ? h * vdim + d : d]);
     const float gv = Elem<T>::load(gate[(cell / heads) * gate_stride + (int64_t)h * vdim + d]);
     const float act = plain_sigmoid ? 1.0f / (1.0f + expf(-gv)) : silu<T>(gv);
-    y[cell * vdim + d] = Elem<T>::store(src[d] * r * wv * act);
+    y[cell * vdim + d] = Elem<T>::store((den ? src[d] / under : src[d]) * r * wv * act);
   }
 }
 
@@ -719,7 +725,7 @@ extern "C" int holon_memory_scan(const void* r, const void* k, const void* v, co
 
 extern "C" int holon_gated_out(const float* o, const void* gate, const void* weight, void* y, int tokens, int heads,
                                int vdim, int per_head, float eps, int dtype, int64_t gate_stride, int plain_sigmoid,
-                               void* stream) {
+                               const float* den, void* stream) {
   HOLON_CHECK(tokens >= 0 && heads > 0 && vdim > 0 && gate_stride >= (int64_t)heads * vdim,
               "gated_out: %d heads of %d, gates %lld apart", heads, vdim, (long long)gate_stride);
   const int64_t cells = (int64_t)tokens * heads;
@@ -727,7 +733,7 @@ extern "C" int holon_gated_out(const float* o, const void* gate, const void* wei
   HOLON_CHECK((cells + 3) / 4 <= 0x7fffffff, "gated_out: %lld cells exceed one launch", (long long)cells);
   BY_DTYPE(dtype, (gated_out_kernel<T><<<(unsigned)((cells + 3) / 4), 256, 0, (hipStream_t)stream>>>(
                       o, (const T*)gate, (const T*)weight, (T*)y, cells, heads, vdim, per_head, eps, gate_stride,
-                      plain_sigmoid)));
+                      plain_sigmoid, den)));
   HOLON_LAUNCH_OK();
   return 0;
 }

@@ -109,27 +109,31 @@ def _delta_scan_hip(launch, qn, kn, qkv, beta, g, state, slots, starts, query_st
     return out
 
 
-def gated_out_plain(o, gate, weight, per_head_weight, eps, out_dtype, act="silu"):
+def gated_out_plain(o, gate, weight, per_head_weight, eps, out_dtype, act="silu", den=None):
     """o [T, H, V] float32 -> [T, H V]: each head's o divided by its root mean square (eps inside the root), times
     `weight` ([V], shared by the heads, or [H V] with `per_head_weight`), times act(gate [T, H V]); `act` is "silu"
-    or "sigmoid". The gates may be columns of a wider tensor (rows further apart than H V)."""
+    or "sigmoid". The gates may be columns of a wider tensor (rows further apart than H V). `den` [T, H] float32 or
+    None: every head's o is divided by it first."""
     t, heads, vdim = o.shape
+    if den is not None:
+        o = o / den[..., None]
     y = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps)
     y = y * (weight.float().view(heads, vdim) if per_head_weight else weight.float())
     gf = gate.float().reshape(t, heads, vdim)
     return (y * (gf if act == "silu" else 1.0) * torch.sigmoid(gf)).view(t, heads * vdim).to(out_dtype)
 
 
-def _gated_out_hip(launch, o, gate, weight, per_head_weight, eps, out_dtype, act="silu"):
+def _gated_out_hip(launch, o, gate, weight, per_head_weight, eps, out_dtype, act="silu", den=None):
     t, heads, vdim = o.shape
     _need(o.is_cuda and o.is_contiguous() and o.dtype == torch.float32 and gate.dtype in _DT and gate.dim() == 2
           and tuple(gate.shape) == (t, heads * vdim) and gate.stride(1) == 1 and (t <= 1 or gate.stride(0) >= heads * vdim)
           and weight.is_contiguous() and weight.dtype == gate.dtype
           and weight.numel() == (heads * vdim if per_head_weight else vdim) and out_dtype == gate.dtype
-          and act in ("silu", "sigmoid"), "gated_out: shapes do not fit")
+          and act in ("silu", "sigmoid") and (den is None or (den.dtype == torch.float32 and den.is_contiguous()
+                                                  and tuple(den.shape) == (t, heads))), "gated_out: shapes do not fit")
     y = torch.empty((t, heads * vdim), dtype=out_dtype, device=o.device)
     launch(o.data_ptr(), gate.data_ptr(), weight.data_ptr(), y.data_ptr(), t, heads, vdim, int(per_head_weight),
-           float(eps), _DT[out_dtype], gate.stride(0) if t > 1 else heads * vdim, int(act == "sigmoid"))
+           float(eps), _DT[out_dtype], gate.stride(0) if t > 1 else heads * vdim, int(act == "sigmoid"), _ptr(den))
     return y
 
 
@@ -243,7 +247,7 @@ register_kernel(KernelOp("delta_scan", delta_scan_plain, "holon_delta_scan",
                          [_P, _P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P],
                          _delta_scan_hip))
 register_kernel(KernelOp("gated_out", gated_out_plain, "holon_gated_out",
-                         [_P, _P, _P, _P, _I, _I, _I, _I, _F, _I, ctypes.c_int64, _I], _gated_out_hip))
+                         [_P, _P, _P, _P, _I, _I, _I, _I, _F, _I, ctypes.c_int64, _I, _P], _gated_out_hip))
 register_kernel(KernelOp("shift_mix", shift_mix_plain, "holon_shift_mix",
                          [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I], _shift_mix_hip))
 register_kernel(KernelOp("decay_lora", decay_lora_plain, "holon_decay_lora", [_P, _P, _P, _P, _I, _I, _I, _I],

@@ -437,19 +437,18 @@ def test_kernels_against_their_plain_forms(dtype):
         c2 = kernel_op("latent_prepare").plain(both, q_rank, qw, cw, 1e-6, pg2, wp, wo, page)
         assert _rel(c1, c2) < tol and _rel(pg1, pg2) < tol
     for heads, d, v in ((4, 48, 48), (2, 16, 40), (3, 64, 8), (1, 128, 20), (2, 200, 16)):     # the memory's scan
-        hd, hv, copies = heads * d, heads * v, -(-v // 8)
+        hd, hv, copies = heads * d, heads * v, -(-(v + 1) // 8)
         width = -(-(2 * hd + 2 * hv + 2 * heads) // 16) * 16
         proj = rn(43, width).to(dtype)
         proj[:, 2 * hd + 2 * hv:] *= 3
         gb = rn(2 * heads)
-        state = [rn(5, heads, d, v), rn(5, heads, 1, d).expand(5, heads, copies, d).contiguous(),
-                 rn(5, heads, 1).expand(5, heads, copies).contiguous()]
+        state = [rn(5, heads, d, v + 1), rn(5, heads, 1).expand(5, heads, copies).contiguous()]
         st1, st2 = [s.clone() for s in state], [s.clone() for s in state]
         rows = (torch.tensor([3, 0, 4], dtype=torch.int32, device=dev), torch.tensor([0, 9, 2], dtype=torch.int32, device=dev),
                 torch.tensor([0, 37, 38, 43], dtype=torch.int32, device=dev))
-        o1 = k.mlstm_scan(proj, 0, hd, 2 * hd, 2 * hd + 2 * hv, gb, 12.0, *st1, *rows, 3, heads, d, v)
-        o2 = kernel_op("mlstm_scan").plain(proj, 0, hd, 2 * hd, 2 * hd + 2 * hv, gb, 12.0, *st2, *rows, 3, heads, d, v)
-        assert _rel(o1, o2) < 1e-5 and all(_rel(a, b) < 1e-5 for a, b in zip(st1, st2))
+        o1, u1 = k.mlstm_scan(proj, 0, hd, 2 * hd, 2 * hd + 2 * hv, gb, 12.0, *st1, *rows, 3, heads, d, v)
+        o2, u2 = kernel_op("mlstm_scan").plain(proj, 0, hd, 2 * hd, 2 * hd + 2 * hv, gb, 12.0, *st2, *rows, 3, heads, d, v)
+        assert _rel(o1, o2) < 1e-5 and _rel(u1, u2) < 1e-5 and all(_rel(a, b) < 1e-5 for a, b in zip(st1, st2))
         # long rows in pieces of 128 tokens: a row of 700 from a carried state, one of 300 from zero, a decode row
         long = rn(1001, width).to(dtype)
         long[:, 2 * hd + 2 * hv:] *= 3
@@ -457,12 +456,12 @@ def test_kernels_against_their_plain_forms(dtype):
                 torch.tensor([0, 700, 1000, 1001], dtype=torch.int32, device=dev))
         cut = (128, 6, torch.tensor([0, 6, 9], dtype=torch.int32, device=dev), 10)
         st3, st4 = [s.clone() for s in state], [s.clone() for s in state]
-        o3 = k.mlstm_scan(long, 0, hd, 2 * hd, 2 * hd + 2 * hv, gb, 12.0, *st3, *rows, 3, heads, d, v, cut)
-        o4 = kernel_op("mlstm_scan").plain(long, 0, hd, 2 * hd, 2 * hd + 2 * hv, gb, 12.0, *st4, *rows, 3, heads, d, v)
-        assert _rel(o3, o4) < 2e-5 and all(_rel(a, b) < 2e-5 for a, b in zip(st3, st4))
+        o3, u3 = k.mlstm_scan(long, 0, hd, 2 * hd, 2 * hd + 2 * hv, gb, 12.0, *st3, *rows, 3, heads, d, v, cut)
+        o4, u4 = kernel_op("mlstm_scan").plain(long, 0, hd, 2 * hd, 2 * hd + 2 * hv, gb, 12.0, *st4, *rows, 3, heads, d, v)
+        assert _rel(o3 / u3[..., None], o4 / u4[..., None]) < 2e-5 and all(_rel(a, b) < 2e-5 for a, b in zip(st3, st4))
         gate, wn = proj[:, 2 * hd + hv: 2 * hd + 2 * hv], rn(hv).to(dtype)
-        assert _rel(k.gated_out(o1, gate, wn, True, 1e-6, dtype, act="sigmoid"),
-                    kernel_op("gated_out").plain(o1, gate, wn, True, 1e-6, dtype, act="sigmoid")) < tol
+        assert _rel(k.gated_out(o1, gate, wn, True, 1e-6, dtype, act="sigmoid", den=u1),
+                    kernel_op("gated_out").plain(o1, gate, wn, True, 1e-6, dtype, act="sigmoid", den=u1)) < tol
 
 
 @pytest.mark.gpu
