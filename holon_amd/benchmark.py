@@ -134,8 +134,8 @@ def relanex_config(z: dict, window: int = 1024) -> dict:
             return {"type": "attention", "mlp": mlp,
                     "mixer": {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["dim"],
                               "scale": z["dim"] ** -0.5,
-                              "rot": {"dims": z["dim"] // 2, "base": 250000.0,
-                                      "scaling": {"factor": 4.0, "original": 2048, "fast": 32.0, "slow": 1.0}}}}
+                              "rot": {"dims": z["dim"] // 2, "base": 1e6,
+                                      "scaling": {"factor": 8.0, "original": 4096, "fast": 16.0, "slow": 2.0}}}}
         if i % 4 == 3:
             return {"type": "mlstm", "mlp": mlp, "mixer": {"heads": z["width"] // 128, "dim": 128, "vdim": 128,
                                                           "gate_cap": 15.0}}
@@ -143,7 +143,7 @@ def relanex_config(z: dict, window: int = 1024) -> dict:
                 "mixer": {"heads": z["heads"], "dim": z["dim"], "vdim": z["dim"], "q_rank": 768, "kv_rank": 256,
                           "mask": {"size": window}, "scale": z["dim"] ** -0.5}}
     return {"architecture": "Relanex", "width": z["width"], "vocab": z["vocab"], "norm": {"eps": 1e-6},
-            "residual_mult": 0.7, "layers": [layer(i) for i in range(z["layers"])]}
+            "residual_mult": 0.5, "layers": [layer(i) for i in range(z["layers"])]}
 
 
 def design_cache_bytes(name: str, cfg_json: dict, z: dict, item: int, batch: int, context: int) -> int:

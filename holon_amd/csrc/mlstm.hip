@@ -1,6 +1,6 @@
 // The matrix memory of xLSTM (mLSTM) along each row's tokens. Per (row, head): a matrix S [D, V], a vector n [D] and a
-// running maximum m, float32, carried in the request's slot (a row that starts at position 0 starts from S = 0, n = 0,
-// m = 0 whatever the slot holds). With log gates i and f of the token:
+// running maximum m, float32, carried in the request's slot (a row that starts at position 0 starts from S = 0, n = 0
+// and a maximum of 0, whatever the slot holds). With log gates i and f of the token:
 //   m' = max(f + m, i);  S' = exp(f + m - m') S + exp(i - m') k v^T;  n' = exp(f + m - m') n + exp(i - m') k
 //   o = S'^T q / (max(|n' . q|, exp(-m')) + 1e-6)
 // The gates come as pre-activations a of a projection and a bias: i = cap tanh((a_i + b_i) / cap),

@@ -1,5 +1,5 @@
 // Softmax attention over a paged cache whose keys and values may differ in width, with an optional sliding window and an
-// optional sink (a number per head that stands in the denominator and has no key or value). The general kernel: any
+// optional sink (one scalar per head whose exponential joins the normaliser; nothing is read from the cache for it). The general kernel: any
 // element type, any sizes.
 //
 // A page of one site holds P tokens: keys [Hkv, P, D] (a token's key is a row), then values [Hkv, V, P] (transposed

@@ -5,7 +5,8 @@ always 1); along a row's tokens, with log gates i and f:
     m' = max(f + m, i);   S' = exp(f + m - m') S + exp(i - m') k v^T;   n' likewise with k alone
     o = S'^T q / (max(|n' . q|, exp(-m')) + 1e-6)
 
-m starts at 0 (not at minus infinity), S and n at zero. The gates are capped, i = cap tanh(a_i / cap) and
+S and n begin as zeros, and the running maximum begins at 0 as well, so a sequence's first token is already
+compared with 0. The gates are capped, i = cap tanh(a_i / cap) and
 f = logsigmoid(cap tanh(a_f / cap)), with a = W x + b; q is scaled by D^-0.5. Each head's o is divided by its root
 mean square, multiplied by `norm` (a weight over all heads' values) and by sigmoid(W_g x), and projected out. One
 product yields q, k, v, the output gate and both gates' pre-activations; gates, decays and the recurrence are float32.

@@ -72,7 +72,7 @@ ONLY_LATENT = {"architecture": "Relanex", "width": 48, "vocab": 90, "norm": {"ep
                "layers": [latent(4, 12, 20, 16, 24, 9, 0.3), latent(2, 16, 8, 32, 8, 20, 0.25)]}
 ONLY_MLSTM = {"architecture": "Relanex", "width": 48, "vocab": 90, "norm": {"eps": 1e-6}, "residual_mult": 0.8,
               "layers": [mlstm(4, 24, 12, 10.0), mlstm(3, 16, 16, 3.0)]}
-ONLY_FFN = {"architecture": "Relanex", "width": 48, "vocab": 90, "norm": {"eps": 1e-6}, "residual_mult": 0.7,
+ONLY_FFN = {"architecture": "Relanex", "width": 48, "vocab": 90, "norm": {"eps": 1e-6}, "residual_mult": 0.9,
             "loop": {"start": 0, "stop": 1, "times": 2}, "layers": [latent(1, 8, 8, 8, 8, 1, 1.0, ff=80)]}
 
 
