@@ -14,6 +14,22 @@ class ConfigError(ValueError):
     """config.json is missing a key, or asks for something this architecture does not do."""
 
 
+def config_value(c: Mapping[str, Any], path: str, kind=None):
+    """c["a"]["b"] for path "a.b"; a missing key is a ConfigError that names the path."""
+    at: Any = c
+    for key in path.split("."):
+        if not isinstance(at, Mapping) or key not in at:
+            raise ConfigError(f"config.json lacks `{path}`")
+        at = at[key]
+    if kind is int and (not isinstance(at, int) or isinstance(at, bool) or at < 1):
+        raise ConfigError(f"`{path}` must be a positive integer, got {at!r}")
+    if kind is float:
+        if not isinstance(at, (int, float)) or isinstance(at, bool):
+            raise ConfigError(f"`{path}` must be a number, got {at!r}")
+        at = float(at)
+    return at
+
+
 def eos_ids(*sources: Mapping[str, Any] | None) -> tuple[int, ...]:
     """The union of `eos_token_id` (an int or a list) over config.json and generation_config.json
     (std/holon_std/weights/hf/source.py:62-66)."""

@@ -16,9 +16,9 @@ from collections.abc import Mapping
 from typing import Any
 
 from ..config.model import ConfigError, eos_ids
+from ..config.model import config_value as _get
 from ..registry import register_architecture
-from ..spec import LayerSpec, ModelSpec, PartRef, WeightRule
-from .tolurax import _get, run_order
+from ..spec import LayerSpec, ModelSpec, PartRef, WeightRule, looped_order
 
 NAME = "Relanex"
 MIXERS = ("attention", "latent_attention", "mlstm")
@@ -143,7 +143,7 @@ def recipe(c: RelanexConfig) -> ModelSpec:
         ffn = PartRef("ffn", "swiglu", inter=mlp["ff"]) if mlp else None
         block = PartRef("block", "sandwich32", scale=c.residual_mult, reentry=bool(c.loop) and i == c.loop[0])
         layers.append(LayerSpec(block=block, mixer=mixer, ffn=ffn, norm=norm))
-    return ModelSpec(hidden=c.width, vocab=c.vocab, layers=tuple(layers), order=run_order(len(layers), c.loop),
+    return ModelSpec(hidden=c.width, vocab=c.vocab, layers=tuple(layers), order=looped_order(len(layers), c.loop),
                      embed=PartRef("embed", "table", norm=norm), norm=norm, head=PartRef("head", "linear", tied=False),
                      rules=_rules(), eos_token_ids=c.eos_token_ids)
 

@@ -16,26 +16,12 @@ from collections.abc import Mapping
 from typing import Any
 
 from ..config.model import ConfigError, eos_ids
+from ..config.model import config_value as _get
 from ..registry import register_architecture
-from ..spec import LayerSpec, ModelSpec, PartRef, Run, WeightRule
+from ..spec import LayerSpec, ModelSpec, PartRef, WeightRule
+from ..spec import looped_order as run_order
 
 NAME = "Tolurax"
-
-
-def _get(c: Mapping[str, Any], path: str, kind=None):
-    """c["a"]["b"] for path "a.b"; a missing key is a ConfigError that names the path."""
-    at: Any = c
-    for key in path.split("."):
-        if not isinstance(at, Mapping) or key not in at:
-            raise ConfigError(f"config.json lacks `{path}`")
-        at = at[key]
-    if kind is int and (not isinstance(at, int) or isinstance(at, bool) or at < 1):
-        raise ConfigError(f"`{path}` must be a positive integer, got {at!r}")
-    if kind is float:
-        if not isinstance(at, (int, float)) or isinstance(at, bool):
-            raise ConfigError(f"`{path}` must be a number, got {at!r}")
-        at = float(at)
-    return at
 
 
 @dataclasses.dataclass(frozen=True)
@@ -138,15 +124,6 @@ def _rules(loop_start: int | None) -> tuple[WeightRule, ...]:
     rules += [WeightRule(f"l{{i}}.mix.right.{s}", f"{mix}right.{s}.weight") for s in ("r", "k", "v", "g", "o")]
     rules += [WeightRule(f"l{{i}}.mix.right.{s}", f"{mix}right.{s}") for s in ("w1", "w2", "w0", "u", "norm")]
     return tuple(rules)
-
-
-def run_order(n_layers: int, loop: tuple[int, int, int] | None) -> tuple[Run, ...]:
-    """Every layer once, the loop's range `times` times in a row; every run keeps a cache of its own."""
-    if not loop:
-        return tuple(Run(i) for i in range(n_layers))
-    start, stop, times = loop
-    order = list(range(start)) + list(range(start, stop)) * times + list(range(stop, n_layers))
-    return tuple(Run(i) for i in order)
 
 
 def recipe(c: ToluraxConfig) -> ModelSpec:

@@ -118,3 +118,12 @@ class ModelSpec:
 def in_order(n_layers: int) -> tuple[Run, ...]:
     """Every layer once, first to last."""
     return tuple(Run(i) for i in range(n_layers))
+
+
+def looped_order(n_layers: int, loop: tuple[int, int, int] | None) -> tuple[Run, ...]:
+    """Every layer once, the loop's range `times` times in a row; every run keeps a cache of its own."""
+    if not loop:
+        return tuple(Run(i) for i in range(n_layers))
+    start, stop, times = loop
+    order = list(range(start)) + list(range(start, stop)) * times + list(range(stop, n_layers))
+    return tuple(Run(i) for i in order)
