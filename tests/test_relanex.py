@@ -369,6 +369,65 @@ def test_greedy_generation_through_the_engine(folders, dtype, device):
     engine.close()
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("name,dtype", [("A-sharp", "float32"), ("A-sharp", "bfloat16"), ("D-sharp", "float32")])
+def test_graph_replays_equal_eager_steps(folders, name, dtype):
+    """Decode steps replayed from HIP graphs give the tokens of eager steps, over many replays with the program's own
+    eager work (prompt steps, sampling, host synchronisation) between them, while the batch shrinks through the
+    buckets, pages are taken and given back and windows pass. (On the matrix-core attention path a replayed step cuts
+    a row's keys over waves as its length bucket asks, an eager one as the row's length does, so the two differ by
+    rounding: that path has the test below.)"""
+    from holon_amd.config import EngineConfig, SamplingParams
+    from holon_amd.engine.engine import Engine
+    vocab = MODELS[name][0]["vocab"]
+    prompts = [H.random_ids(n, vocab, 80 + n) for n in (3, 17, 8, 25, 40, 1)]
+    outs = {}
+    for graphs in (False, True):
+        engine = Engine(EngineConfig(model=str(folders[name]), device="cuda", dtype=dtype, page_size=16, max_seqs=6,
+                                     max_model_len=160, max_step_tokens=64, graphs=graphs, cache_tokens=960))
+        rids = [engine.add(p, SamplingParams(temperature=0.0 if i % 2 else 0.7, seed=5, max_tokens=60 + 7 * i,
+                                             ignore_eos=True)) for i, p in enumerate(prompts)]
+        got = {r: [] for r in rids}
+        while engine.has_work():
+            for d in engine.step():
+                got[d.rid].extend(d.token_ids)
+        outs[graphs] = [got[r] for r in rids]
+        engine.cache.check()
+        if graphs:
+            assert engine.runner.graph_replays > 20 and len(engine.runner.graphs) >= 3
+        engine.close()
+    assert outs[True] == outs[False]
+
+
+@pytest.mark.gpu
+def test_graph_replays_on_the_matrix_core_path(folders):
+    """bfloat16 at head sizes the matrix-core kernels serve (the sink and the window among them): logits of decode
+    steps replayed from graphs, two requests side by side and then one alone, against eager steps: as near the plain
+    model as they are, and no further from each other than rounding puts them."""
+    from holon_amd.engine.loading import load_model
+    from holon_amd.engine.replay import Replayer
+    folder = folders["D-sharp"]
+    vocab = MODELS["D-sharp"][0]["vocab"]
+    ids, other = H.random_ids(150, vocab, 7), H.random_ids(90, vocab, 8)
+    want = _plain(str(folder)).logits(ids)[20:]
+    outs = {}
+    for graphs in (False, True):
+        rep = Replayer(load_model(folder, device="cuda", dtype="bfloat16", page_size=16, max_seqs=6, max_model_len=160,
+                                  max_step_tokens=64, cache_tokens=960, graphs=graphs))
+        rep.step([{"id": "a", "tokens": ids[:20], "want": []}, {"id": "b", "tokens": other[:33], "want": []}])
+        rows = []
+        for p in range(20, 150):
+            entries = [{"id": "a", "tokens": [ids[p]], "want": [0]}]
+            if 13 + p < 90:
+                entries.append({"id": "b", "tokens": [other[13 + p]], "want": [0]})
+            rows.append(rep.step(entries)[0].float().cpu().clone())
+        outs[graphs] = torch.stack(rows)
+        assert rep.runner.graph_replays > 100 if graphs else rep.runner.graph_replays == 0
+        assert H.rel_rms(outs[graphs], want) < 0.02
+    apart = (outs[True] - outs[False]).square().mean(-1).sqrt() / outs[False].square().mean().sqrt()
+    assert apart.max().item() < 0.03
+
+
 # -- the HIP kernels alone, each against its plain form --------------------------------------------------------------
 def _rel(a, b):
     return H.rel_rms(a.float(), b.float())
